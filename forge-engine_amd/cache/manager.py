@@ -31,6 +31,21 @@ class CacheGroup:
     window: int | None
     slots: tuple[int, ...]  # cache slots (schedule indices that write) in this group
     value_dim: int = -1     # width of a value row (-1: head_dim; 0: the group holds keys only)
+    chunk: int | None = None   # keys are read within runs of this many positions only
+
+    @property
+    def gives_back(self) -> bool:
+        """Whether pages of a live request go back to the pool as it grows."""
+        return self.window is not None or self.chunk is not None
+
+    def first_needed(self, next_position: int) -> int:
+        """The first key that the token at ``next_position`` or any later one can read."""
+        first = 0
+        if self.window is not None:
+            first = max(first, next_position - self.window + 1)
+        if self.chunk is not None:
+            first = max(first, next_position // self.chunk * self.chunk)
+        return first
 
     @property
     def value_width(self) -> int:
@@ -58,11 +73,11 @@ def plan_groups(needs: list[CacheNeeds], schedule) -> tuple[list[CacheGroup], di
         paged = needs[index].paged
         if paged is None or call.cache != index:
             continue
-        by_key.setdefault((paged.kv_heads, paged.head_dim, paged.window, paged.value_width), []).append(index)
+        by_key.setdefault((paged.kv_heads, paged.head_dim, paged.window, paged.value_width, paged.chunk), []).append(index)
     groups = []
     where: dict[int, tuple[int, int]] = {}
     for g, (key, slots) in enumerate(by_key.items()):
-        groups.append(CacheGroup(g, key[0], key[1], key[2], tuple(slots), key[3]))
+        groups.append(CacheGroup(g, key[0], key[1], key[2], tuple(slots), key[3], key[4]))
         for j, slot in enumerate(slots):
             where[slot] = (g, j)
     for index, call in enumerate(schedule):
@@ -75,6 +90,8 @@ def plan_groups(needs: list[CacheNeeds], schedule) -> tuple[list[CacheGroup], di
                 raise ValueError(f"schedule entry {index} reads a cache of another geometry")
             # the owner's window decides which pages go back: a reader that looks further back
             # would read pages that are no longer the request's
+            if owner.chunk != paged.chunk and owner.chunk is not None:
+                raise ValueError(f"schedule entry {index} reads cache slot {call.cache}, which keeps runs of {owner.chunk} keys only")
             if owner.window is not None and (paged.window is None or paged.window > owner.window):
                 raise ValueError(
                     f"schedule entry {index} looks back {paged.window or 'without limit'} but reads cache slot "
@@ -137,10 +154,11 @@ class CacheManager:
         whole = self.blocks_for(total_tokens)
         bounds = []
         for group in self.groups:
-            if group.window is None or step_tokens is None:
+            if not group.gives_back or step_tokens is None:
                 bounds.append(whole)
             else:
-                bounds.append(min(whole, self.blocks_for(group.window - 1 + step_tokens) + 1))
+                reach = min(r for r in (group.window, group.chunk) if r is not None)
+                bounds.append(min(whole, self.blocks_for(reach - 1 + step_tokens) + 1))
         return bounds
 
     @property
@@ -188,11 +206,11 @@ class CacheManager:
             raise ValueError(f"request '{request_id}' has no pages for length {new_length}")
         entry.length = new_length
         for g, group in enumerate(self.groups):
-            if group.window is None:
+            if not group.gives_back:
                 continue
-            # the next token sits at position new_length and reads keys > new_length - window
-            first_needed = max(0, new_length - group.window + 1)
-            keep_from = first_needed // self.block_size
+            # the next token sits at position new_length and reads keys > new_length - window,
+            # or of its own run of positions only
+            keep_from = group.first_needed(new_length) // self.block_size
             table = entry.tables[g]
             passed = [b for b in range(entry.first_block[g], min(keep_from, len(table)))]
             if passed:
@@ -203,7 +221,7 @@ class CacheManager:
 
     def commit_single_tokens(self, entries: list[RequestCache]) -> None:
         """``commit`` for requests that each grew by one token (the decode step)."""
-        windowed = any(group.window is not None for group in self.groups)
+        windowed = any(group.gives_back for group in self.groups)
         for entry in entries:
             if windowed:
                 self.commit(entry.request_id, entry.length + 1)

@@ -10,12 +10,15 @@ from typing import Any, Mapping
 class PagedKV:
     """Keys and values in pages.  ``window`` None: every key is kept; else only
     the last ``window`` keys of a request are ever read again, and pages that
-    the window has passed go back to the pool."""
+    the window has passed go back to the pool.  ``chunk``: a token reads keys of its own run of
+    ``chunk`` positions only (runs counted from position 0), so pages that lie wholly before the
+    run of a request's next token go back as well."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None   # width of a value row: None, as wide as a key; 0: keys only, no value pages at all
+    chunk: int | None = None
 
     @property
     def value_width(self) -> int:

@@ -2,7 +2,8 @@
 
 from .engine import EngineConfig, SchedulerConfig
 from .model import ConfigError, ModelConfig, load_model_config
+from .mazanex import MazanexConfig
 from .qwen3 import Qwen3Config
 
-__all__ = ["ConfigError", "EngineConfig", "ModelConfig", "Qwen3Config", "SchedulerConfig",
+__all__ = ["ConfigError", "EngineConfig", "MazanexConfig", "ModelConfig", "Qwen3Config", "SchedulerConfig",
            "load_model_config"]

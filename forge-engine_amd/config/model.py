@@ -60,9 +60,12 @@ def read_config_json(path: str | Path) -> dict[str, Any]:
 
 def architecture_name(raw: dict[str, Any]) -> str:
     names = raw.get("architectures")
-    if not isinstance(names, list) or not names or not isinstance(names[0], str):
-        raise ConfigError("config.json must name the model under 'architectures'")
-    return names[0]
+    if isinstance(names, list) and names and isinstance(names[0], str):
+        return names[0]
+    single = raw.get("architecture")     # some designs name themselves with one string
+    if isinstance(single, str) and single:
+        return single
+    raise ConfigError("config.json must name the model under 'architectures' (a list) or 'architecture'")
 
 
 def load_model_config(source: str | Path | dict[str, Any]) -> ModelConfig:

@@ -48,6 +48,9 @@ def load_model(folder: str | Path, *, dtype="bfloat16", device="cuda:0") -> tupl
     """config.json chooses the model class; the safetensors files fill it."""
     folder = Path(folder)
     config = load_model_config(folder)
+    if hasattr(config, "with_tensor_shapes"):     # a design some of whose sizes only the tensors' shapes give
+        from ..weights.loader import checkpoint_shapes
+        config = config.with_tensor_shapes(checkpoint_shapes(folder))
     model = build_model(config, dtype=dtype, device=device)
     load_weights(model, folder, device=model.ctx.device, dtype=model.ctx.dtype)
     return config, model

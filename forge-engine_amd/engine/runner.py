@@ -369,7 +369,7 @@ class ModelRunner:
         self.graph_replays += 1
         cache.commit_single_tokens(records)
         self.steps_run += 1
-        if not any(group.window is not None for group in cache.groups):   # a window gives pages back as it moves
+        if not any(group.gives_back for group in cache.groups):   # a window gives pages back as it moves
             room = min(len(table) * self.block_size - record.length for record in records for table in record.tables)
             self._steady = _SteadyDecode(tuple(e.request_id for e in entries), records, slot, room)
         return slot.logits

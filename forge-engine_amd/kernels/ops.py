@@ -981,3 +981,353 @@ def sample_filtered_rows(logits: Tensor, params: Tensor, tokens: Tensor, status:
 
 
 LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")
+
+
+# ------------------------------------------------- ops on the stream, beside the matrix products
+
+def cast_rows(h: Tensor, dtype) -> Tensor:
+    """The stream in the compute dtype (itself when that is float32)."""
+    _gpu(h, "h")
+    return h if h.dtype == dtype else h.to(dtype)
+
+
+def _sequences(cu_q: Tensor, state_slots: Tensor, num_seqs: int) -> None:
+    _gpu(cu_q, "cu_q", torch.int32)
+    _gpu(state_slots, "state_slots", torch.int32)
+    if num_seqs < 1 or cu_q.numel() != num_seqs + 1 or state_slots.numel() != num_seqs:
+        raise KernelError("cu_q and state_slots do not match the number of sequences")
+
+
+def _parts_of(update: Tensor, rows: int, width: int, name: str) -> int:
+    _gpu(update, name, torch.float32)
+    if update.shape == (rows, width):
+        return 1
+    if update.dim() == 3 and update.shape[1:] == (rows, width) and 1 <= update.shape[0] <= 64:
+        return update.shape[0]
+    raise KernelError(f"{name} must be [{rows}, {width}] or [parts <= 64, {rows}, {width}], got {tuple(update.shape)}")
+
+
+def token_shift(x: Tensor, weights: Tensor, state: Tensor, cu_q: Tensor, token_seq: Tensor, state_slots: Tensor, *,
+                num_seqs: int, out_dtype) -> Tensor:
+    """out[s, t] = x[t] + (x'[t] - x[t]) * weights[s]: x' is the row before within the token's
+    sequence, and for a sequence's first token of the step the row that ``state`` keeps for its slot
+    (zeros for a request's first token); afterwards ``state`` holds every sequence's last row.
+    x [T, W] float32 or bfloat16, weights float32 [n, W], state float32 [slots, W]; out [n, T, W]."""
+    _gpu(x, "x")
+    _gpu(weights, "weights", torch.float32)
+    _gpu(state, "state", torch.float32)
+    _gpu(token_seq, "token_seq", torch.int32)
+    _sequences(cu_q, state_slots, num_seqs)
+    tokens, width = x.shape
+    if weights.dim() != 2 or weights.shape[1] != width or not 1 <= weights.shape[0] <= 8:
+        raise KernelError(f"weights must be [1..8, {width}], got {tuple(weights.shape)}")
+    if state.dim() != 2 or state.shape[1] != width or token_seq.numel() != tokens:
+        raise KernelError("state must be [slots, width] and token_seq hold one entry per token")
+    out = torch.empty((weights.shape[0], tokens, width), dtype=out_dtype, device=x.device)
+    _call("stream_ops", "fe_token_shift", _ptr(x), c_int(_code(x.dtype)), _ptr(weights), _ptr(state), _ptr(cu_q),
+          _ptr(token_seq), _ptr(state_slots), _ptr(out), c_int(_code(out.dtype)), c_int(tokens), c_int(width),
+          c_int(weights.shape[0]), c_int(state.shape[0]), _stream())
+    _call("stream_ops", "fe_save_last_rows", _ptr(x), c_int(_code(x.dtype)), _ptr(state), _ptr(cu_q), _ptr(state_slots),
+          c_int(num_seqs), c_int(width), c_int(state.shape[0]), c_int(tokens), _stream())
+    return out
+
+
+def rmsnorm_update(h: Tensor, update: Tensor, weight: Tensor, eps: float, out: Tensor | None = None) -> Tensor | None:
+    """h += u * rsqrt(mean(u^2) + eps) * weight, u the update (float32, [parts, T, W] added up in
+    order first); all float32.  ``out`` (compute dtype [T, W]) receives the new h as well."""
+    _gpu(h, "h", torch.float32)
+    _gpu(weight, "weight", torch.float32)
+    rows, width = h.shape
+    parts = _parts_of(update, rows, width, "update")
+    if weight.shape != (width,):
+        raise KernelError(f"weight must be [{width}]")
+    if out is not None:
+        _gpu(out, "out")
+        if out.shape != h.shape:
+            raise KernelError("out must have the stream's shape")
+    if not eps > 0.0:
+        raise KernelError("eps must be positive")
+    _call("stream_ops", "fe_rmsnorm_update", _ptr(h), _ptr(update), c_int(parts), c_longlong(h.numel()), _ptr(weight),
+          c_float(eps), _ptr(out), c_int(_code(out.dtype) if out is not None else -1), c_int(rows), c_int(width), _stream())
+    return out
+
+
+def rmsnorm_mean(updates, weights: Tensor, eps: float, out: Tensor) -> Tensor:
+    """out = mean over b of u_b * rsqrt(mean(u_b^2) + eps) * weights[b]; float32 (an update may
+    come as [parts, T, W])."""
+    _gpu(out, "out", torch.float32)
+    _gpu(weights, "weights", torch.float32)
+    rows, width = out.shape
+    count = len(updates)
+    if not 1 <= count <= 4 or weights.shape != (count, width):
+        raise KernelError(f"one to four updates with weights [{count}, {width}]")
+    parts = [_parts_of(u, rows, width, f"update {i}") for i, u in enumerate(updates)]
+    pointers = [_ptr(updates[i]) if i < count else _ptr(None) for i in range(4)]
+    counts = [c_int(parts[i] if i < count else 0) for i in range(4)]
+    _call("stream_ops", "fe_rmsnorm_mean", *pointers, *counts, c_int(count), c_longlong(out.numel()), _ptr(weights),
+          c_float(eps), _ptr(out), c_int(rows), c_int(width), _stream())
+    return out
+
+
+def polynorm(z: Tensor, coefficients: Tensor, eps: float, out: Tensor) -> Tensor:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e, N(y) = y * rsqrt(mean(y^2) + eps) over a row; the
+    four numbers float32 on the device; float32 inside."""
+    _gpu(z, "z")
+    _gpu(out, "out", z.dtype)
+    _gpu(coefficients, "coefficients", torch.float32)
+    if z.dim() != 2 or out.shape != z.shape or coefficients.numel() != 4:
+        raise KernelError("z and out must be [T, F] and the coefficients four numbers")
+    _call("stream_ops", "fe_polynorm", _ptr(z), c_int(_code(z.dtype)), _ptr(coefficients), c_float(eps), _ptr(out),
+          c_int(z.shape[0]), c_int(z.shape[1]), _stream())
+    return out
+
+
+def tanh_rows(x: Tensor) -> Tensor:
+    """tanh of every element, in place (float32 inside)."""
+    _gpu(x, "x")
+    _call("stream_ops", "fe_tanh_rows", _ptr(x), c_int(_code(x.dtype)), c_longlong(x.numel()), _stream())
+    return x
+
+
+_ACTS = {"none": 0, "silu": 1, "sigmoid": 2}
+
+
+def _strided_rows(t: Tensor, name: str, width: int) -> int:
+    _gpu(t, name, contiguous=False)
+    if t.dim() != 2 or t.shape[1] != width or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name} must be [T, {width}] with unit inner stride, got {tuple(t.shape)}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), width)
+
+
+def head_norm_gate(o: Tensor, weight: Tensor | None, gate: Tensor | None, out: Tensor, *, heads: int, dim: int,
+                   eps: float, act: str = "none", extra: int = 0, floor: Tensor | None = None) -> Tensor:
+    """out[t, h] = o[t, h, :dim] / rms * weight * act(gate[t, h]) per head, rms over dim (epsilon
+    inside the root).  o float32 [T, heads, dim + extra]; with ``extra`` = 1 the last column is a
+    normaliser n and the head is first divided by max(|n|, floor[t, h]) + 1e-6.  weight float32
+    of heads * dim entries, or of dim entries shared by the heads; gate [T, heads * dim] rows of
+    any stride, in the compute dtype."""
+    _gpu(o, "o", torch.float32)
+    _gpu(out, "out")
+    tokens = o.shape[0]
+    if o.shape != (tokens, heads, dim + extra) or extra not in (0, 1) or out.shape != (tokens, heads * dim):
+        raise KernelError(f"o must be [T, {heads}, {dim + extra}] and out [T, {heads * dim}]")
+    if act not in _ACTS:
+        raise KernelError(f"unknown gate activation '{act}'")
+    weight_len = 0
+    if weight is not None:
+        _gpu(weight, "weight", torch.float32)
+        weight_len = weight.numel()
+        if weight_len not in (dim, heads * dim):
+            raise KernelError(f"weight must hold {dim} or {heads * dim} entries")
+    gate_stride = 0
+    if gate is not None:
+        gate_stride = _strided_rows(gate, "gate", heads * dim)
+        if gate.dtype != out.dtype:
+            raise KernelError("gate must be in the output's dtype")
+    if extra:
+        _gpu(floor, "floor", torch.float32)
+        if floor.shape != (tokens, heads):
+            raise KernelError(f"floor must be [T, {heads}]")
+    _call("stream_ops", "fe_head_norm_gate", _ptr(o), _ptr(weight), c_int(weight_len), _ptr(gate), c_longlong(gate_stride),
+          _ptr(out), c_int(_code(out.dtype)), _ptr(floor if extra else None), c_int(tokens), c_int(heads), c_int(dim),
+          c_int(extra), c_float(eps), c_int(_ACTS[act]), _stream())
+    return out
+
+
+# ------------------------------------------------- short convolution, rotation, unit norm, page write
+
+def conv_rope_norm_write(qkv: Tensor, conv_weight: Tensor | None, conv_state: Tensor | None, inv_freq: Tensor | None,
+                         positions: Tensor, token_seq: Tensor, cu_q: Tensor, state_slots: Tensor, block_table: Tensor,
+                         key_pages: Tensor, value_pages: Tensor, q_out: Tensor, *, num_seqs: int, q_heads: int,
+                         kv_heads: int, head_dim: int, value_dim: int, rotary_dim: int, unit_norm_eps: float | None,
+                         taps: int) -> None:
+    """From the projection's output to queries and cached keys and values in one kernel: a short
+    causal convolution over time on every q, k and v channel (``taps`` > 0: y_t = sum_j c[:, j] *
+    u_(t - taps + 1 + j), rows before the step from ``conv_state`` [slots, taps - 1, channels],
+    which afterwards holds every sequence's last taps - 1 projected rows); rotation of the first
+    ``rotary_dim`` dims of q and k heads (dim i pairs with i + rotary_dim / 2); then q and k heads
+    divided by their root mean square (``unit_norm_eps`` not None); q into ``q_out`` [T, Hq * D],
+    k and v into their pages (values transposed).  float32 inside, one rounding at the stores.
+    qkv [T, >= channels] with any row stride."""
+    channels = (q_heads + kv_heads) * head_dim + kv_heads * value_dim
+    _gpu(qkv, "qkv", contiguous=False)
+    tokens = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.shape[1] < channels or qkv.stride(1) != 1:
+        raise KernelError(f"qkv must be [T, >= {channels}] with unit inner stride")
+    _gpu(q_out, "q_out", qkv.dtype)
+    if q_out.shape != (tokens, q_heads * head_dim):
+        raise KernelError(f"q_out must be [{tokens}, {q_heads * head_dim}]")
+    if taps:
+        _gpu(conv_weight, "conv_weight", torch.float32)
+        _gpu(conv_state, "conv_state", torch.float32)
+        if conv_weight.shape != (channels, taps) or not 2 <= taps <= 8:
+            raise KernelError(f"conv_weight must be [{channels}, taps in 2..8]")
+        if conv_state.dim() != 3 or conv_state.shape[1:] != (taps - 1, channels):
+            raise KernelError(f"conv_state must be [slots, {taps - 1}, {channels}]")
+    if rotary_dim:
+        _gpu(inv_freq, "inv_freq", torch.float32)
+        if inv_freq.shape != (rotary_dim // 2,) or rotary_dim % 2 or rotary_dim > head_dim:
+            raise KernelError(f"inv_freq must be [{rotary_dim // 2}] for an even rotary_dim <= head_dim")
+    if head_dim > 256 or value_dim > 256:
+        raise KernelError("head sizes up to 256")
+    _gpu(positions, "positions", torch.int32)
+    _gpu(token_seq, "token_seq", torch.int32)
+    _sequences(cu_q, state_slots, num_seqs)
+    if positions.numel() != tokens or token_seq.numel() != tokens:
+        raise KernelError("positions and token_seq must have one entry per token")
+    _gpu(block_table, "block_table", torch.int32)
+    _gpu(key_pages, "key_pages", qkv.dtype)
+    _gpu(value_pages, "value_pages", qkv.dtype)
+    if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
+        raise KernelError(f"key pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
+    num_blocks, _, block_size, _ = key_pages.shape
+    if value_pages.shape != (num_blocks, kv_heads, value_dim, block_size):
+        raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {value_dim}, block_size], got {tuple(value_pages.shape)}")
+    if block_table.dim() != 2 or block_table.stride(1) != 1 or block_table.shape[0] < num_seqs:
+        raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+    stride = qkv.stride(0) if tokens > 1 else max(qkv.stride(0), qkv.shape[1])
+    slots = conv_state.shape[0] if taps else 0
+    _call("conv_rope", "fe_conv_rope_norm_write", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride),
+          _ptr(conv_weight if taps else None), _ptr(conv_state if taps else None), _ptr(inv_freq if rotary_dim else None),
+          _ptr(positions), _ptr(token_seq), _ptr(cu_q), _ptr(state_slots), _ptr(block_table), c_int(block_table.stride(0)),
+          _ptr(key_pages), _ptr(value_pages), _ptr(q_out), c_int(tokens), c_int(q_heads), c_int(kv_heads), c_int(head_dim),
+          c_int(value_dim), c_int(rotary_dim), c_float(unit_norm_eps if unit_norm_eps is not None else 0.0),
+          c_int(1 if unit_norm_eps is not None else 0), c_int(taps), c_int(block_size), c_int(num_blocks), c_int(slots),
+          _stream())
+    if taps:
+        _call("conv_rope", "fe_conv_state_update", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(conv_state),
+              _ptr(cu_q), _ptr(state_slots), c_int(num_seqs), c_int(channels), c_int(taps), c_int(slots), c_int(tokens),
+              _stream())
+
+
+def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor, ctx_len: Tensor,
+                     block_table: Tensor, *, num_seqs: int, max_q_len: int, q_heads: int, kv_heads: int, head_dim: int,
+                     value_dim: int, scale: float, window: int | None = None, chunk: int | None = None,
+                     sink: Tensor | None = None, gate: Tensor | None = None) -> Tensor:
+    """Paged grouped-query attention with the masks and softmax forms beyond the causal one: the
+    query at position p reads keys j <= p with j > p - window (``window``) and j >= p - p % chunk
+    (``chunk``); ``sink`` (float32 [Hq]) adds exp(sink_h) to head h's softmax denominator, with
+    no key and no value; values may be of another width than keys; ``gate`` ([T, Hq * Dv] rows of
+    any stride) multiplies the result by sigmoid(gate).  out [T, Hq * Dv].  Scores and softmax
+    float32."""
+    _gpu(q, "q", contiguous=False)
+    _gpu(out, "out", q.dtype)
+    _gpu(key_pages, "key_pages", q.dtype)
+    _gpu(value_pages, "value_pages", q.dtype)
+    _gpu(cu_q, "cu_q", torch.int32)
+    _gpu(ctx_len, "ctx_len", torch.int32)
+    _gpu(block_table, "block_table", torch.int32)
+    tokens = q.shape[0]
+    q_stride = _strided_rows(q, "q", q_heads * head_dim)
+    if out.shape != (tokens, q_heads * value_dim):
+        raise KernelError(f"out must be [{tokens}, {q_heads * value_dim}], got {tuple(out.shape)}")
+    if q_heads % kv_heads or not 1 <= head_dim <= 256 or not 1 <= value_dim <= 256:
+        raise KernelError("query heads must be a multiple of kv heads, head sizes in [1, 256]")
+    if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
+        raise KernelError(f"key pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
+    num_blocks, _, block_size, _ = key_pages.shape
+    if value_pages.shape != (num_blocks, kv_heads, value_dim, block_size):
+        raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {value_dim}, block_size]")
+    if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.shape[0] < num_seqs:
+        raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
+    if block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+    if sink is not None:
+        _gpu(sink, "sink", torch.float32)
+        if sink.shape != (q_heads,):
+            raise KernelError(f"sink must be [{q_heads}]")
+    gate_stride = 0
+    if gate is not None:
+        gate_stride = _strided_rows(gate, "gate", q_heads * value_dim)
+        if gate.dtype != q.dtype:
+            raise KernelError("gate must be in q's dtype")
+    if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
+        raise KernelError("window, chunk and max_q_len must be positive")
+    _call("attention_masked", "fe_masked_attention", _ptr(q), c_int(_code(q.dtype)), c_longlong(q_stride), _ptr(key_pages),
+          _ptr(value_pages), _ptr(out), _ptr(gate), c_longlong(gate_stride), _ptr(sink), _ptr(cu_q), _ptr(ctx_len),
+          _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(q_heads),
+          c_int(kv_heads), c_int(head_dim), c_int(value_dim), c_int(block_size), c_int(num_blocks),
+          c_int(window or 0), c_int(chunk or 0), c_float(scale), c_int(tokens), _stream())
+    return out
+
+
+# ------------------------------------------------- linear recurrences over a matrix state
+
+_DECAY_KINDS = {"none": 0, "exp_neg_exp": 1, "sigmoid_root": 2}
+
+
+def linear_recurrence(q: Tensor, k: Tensor, v: Tensor, out: Tensor, state: Tensor, cu_q: Tensor, state_slots: Tensor, *,
+                      num_seqs: int, max_q_len: int, heads: int, key_dim: int, value_dim: int,
+                      decay: Tensor | None = None, decay_kind: str = "none", decay_bias: Tensor | None = None,
+                      tau: float = 1.0, head_decay: Tensor | None = None, in_scale: Tensor | None = None,
+                      q_scale: float = 1.0, bonus: Tensor | None = None, ones_column: bool = False) -> Tensor:
+    """Per sequence and head, token after token:  S <- diag(a_t) S + b_t k_t v_t^T,  o_t = S^T (q_t *
+    q_scale), with S [key_dim, value_dim] float32 carried in ``state`` [slots, heads, value_dim (+1),
+    key_dim] (value-major) between steps.
+
+    a_t per key channel from ``decay`` (float32 [T, heads * key_dim], before its bias):
+    ``exp_neg_exp`` a = exp(-exp(d + bias)), ``sigmoid_root`` a = sigmoid(d + bias)^(1 / tau); times
+    ``head_decay`` (float32 [T, heads]) where given; b_t = ``in_scale`` [T, heads] or 1.
+    ``bonus`` (float32 [heads * key_dim]): the query reads the state before the token's update plus
+    diag(bonus) k_t v_t^T instead.  ``ones_column``: one more value column fed by v = 1 (a
+    normaliser).  q, k [T, heads * key_dim] and v [T, heads * value_dim] rows of any stride, in the
+    compute dtype; out float32 [T, heads, value_dim (+1)]."""
+    columns = value_dim + (1 if ones_column else 0)
+    tokens = q.shape[0]
+    strides = [_strided_rows(q, "q", heads * key_dim), _strided_rows(k, "k", heads * key_dim),
+               _strided_rows(v, "v", heads * value_dim)]
+    if k.dtype != q.dtype or v.dtype != q.dtype or k.shape[0] != tokens or v.shape[0] != tokens:
+        raise KernelError("q, k and v must share dtype and token count")
+    _gpu(out, "out", torch.float32)
+    _gpu(state, "state", torch.float32)
+    _sequences(cu_q, state_slots, num_seqs)
+    if out.shape != (tokens, heads, columns):
+        raise KernelError(f"out must be [{tokens}, {heads}, {columns}], got {tuple(out.shape)}")
+    if state.dim() != 4 or state.shape[1:] != (heads, columns, key_dim):
+        raise KernelError(f"state must be [slots, {heads}, {columns}, {key_dim}], got {tuple(state.shape)}")
+    if not 1 <= key_dim <= 256:
+        raise KernelError("key sizes up to 256")
+    if decay_kind not in _DECAY_KINDS or (decay is None) != (decay_kind == "none"):
+        raise KernelError("decay and decay_kind go together")
+    for name, t, shape in (("decay", decay, (tokens, heads * key_dim)), ("decay_bias", decay_bias, (heads * key_dim,)),
+                           ("head_decay", head_decay, (tokens, heads)), ("in_scale", in_scale, (tokens, heads)),
+                           ("bonus", bonus, None)):
+        if t is not None:
+            _gpu(t, name, torch.float32)
+            if shape is not None and tuple(t.shape) != shape:
+                raise KernelError(f"{name} must be {shape}, got {tuple(t.shape)}")
+    if bonus is not None and bonus.numel() != heads * key_dim:
+        raise KernelError(f"bonus must hold {heads * key_dim} entries")
+    if decay is not None and decay_bias is None:
+        raise KernelError("a decay comes with its bias")
+    if max_q_len < 1 or not tau > 0.0:
+        raise KernelError("max_q_len and tau must be positive")
+    _call("linear_recurrence", "fe_linear_recurrence", _ptr(q), _ptr(k), _ptr(v), c_int(_code(q.dtype)),
+          c_longlong(strides[0]), c_longlong(strides[1]), c_longlong(strides[2]), _ptr(decay), c_int(_DECAY_KINDS[decay_kind]),
+          _ptr(decay_bias), c_float(tau), _ptr(head_decay), _ptr(in_scale), c_float(q_scale), _ptr(bonus),
+          c_int(1 if ones_column else 0), _ptr(state), c_int(state.shape[0]), _ptr(out), _ptr(cu_q), _ptr(state_slots),
+          c_int(num_seqs), c_int(max_q_len), c_int(heads), c_int(key_dim), c_int(value_dim), c_int(tokens), _stream())
+    return out
+
+
+def mlstm_gate_scan(gates: Tensor, bias: Tensor, cap: float, maximum: Tensor, cu_q: Tensor, state_slots: Tensor,
+                    out: Tensor, *, num_seqs: int, heads: int) -> Tensor:
+    """The stabilised gates of an mLSTM, per sequence and head along the tokens: with i = cap tanh((g_i +
+    b_i) / cap), f = logsigmoid(cap tanh((g_f + b_f) / cap)) and the running maximum m_t = max(f + m_(t-1),
+    i) (``maximum`` [slots, heads] keeps m between steps, 0 for a new request): out[0] = exp(f + m_(t-1) -
+    m_t), out[1] = exp(i - m_t), out[2] = exp(-m_t).  gates float32 [T, 2 heads] (input gates, then forget
+    gates), bias float32 [2 heads], out float32 [3, T, heads]."""
+    _gpu(gates, "gates", torch.float32)
+    _gpu(bias, "bias", torch.float32)
+    _gpu(maximum, "maximum", torch.float32)
+    _gpu(out, "out", torch.float32)
+    _sequences(cu_q, state_slots, num_seqs)
+    tokens = gates.shape[0]
+    if gates.shape != (tokens, 2 * heads) or bias.shape != (2 * heads,) or out.shape != (3, tokens, heads):
+        raise KernelError(f"gates [T, {2 * heads}], bias [{2 * heads}], out [3, T, {heads}]")
+    if maximum.dim() != 2 or maximum.shape[1] != heads or not cap > 0.0:
+        raise KernelError(f"maximum must be [slots, {heads}] and cap positive")
+    _call("linear_recurrence", "fe_mlstm_gate_scan", _ptr(gates), _ptr(bias), c_float(cap), _ptr(maximum),
+          c_int(maximum.shape[0]), _ptr(cu_q), _ptr(state_slots), _ptr(out), c_int(tokens), c_int(num_seqs), c_int(heads),
+          _stream())
+    return out

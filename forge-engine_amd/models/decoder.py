@@ -23,9 +23,10 @@ class DecoderModel:
         self.layers: list[Block] = []
         for spec in plan.layers:
             mixer = build_part("mixer", spec.mixer, ctx)
-            feed_forward = build_part("feed_forward", spec.feed_forward, ctx)
+            feed_forward = None if spec.feed_forward is None else build_part("feed_forward", spec.feed_forward, ctx)
             norms = {role: build_part("norm", norm_spec, ctx) for role, norm_spec in spec.norms.items()}
-            self.layers.append(part_class("block", spec.block)(ctx, mixer, feed_forward, norms))
+            extra = dict(spec.block_params, prefix=spec.prefix) if (spec.block_params or spec.prefix) else {}
+            self.layers.append(part_class("block", spec.block)(ctx, mixer, feed_forward, norms, **extra))
         self.final_norm = build_part("norm", plan.final_norm, ctx)
         self.head = build_part("head", plan.head, ctx)
         if getattr(self.head, "tied", False):
@@ -55,7 +56,7 @@ class DecoderModel:
         """Tensors a checkpoint may hold that the model does not read: the head
         matrix of a model whose head is tied to the embedding."""
         if getattr(self.head, "tied", False):
-            return {self.head.name("weight")}
+            return {self.head.name(getattr(self.head, "leaf", "weight"))}
         return set()
 
     def set_param(self, name: str, tensor: Tensor) -> None:
@@ -91,7 +92,7 @@ class DecoderModel:
 
     def cache_needs(self) -> list[CacheNeeds]:
         """One entry per schedule call (what its mixer asks of the cache)."""
-        return [self.layers[call.layer].mixer.cache_needs() for call in self.schedule]
+        return [self.layers[call.layer].cache_needs() for call in self.schedule]
 
     # --------------------------------------------------------------- running
     def forward(self, batch, cache_views: list[CacheView | None]) -> Tensor:

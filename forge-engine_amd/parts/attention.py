@@ -7,6 +7,19 @@ each query head h over the keys of kv head h // G with scale head_dim^-0.5 and
 the causal mask; output projection.  The keys and values of the step's tokens
 go into their pages first, and attention then reads everything through the
 block table, so a step may hold any portion of any request.
+
+Options beside that (each off by default, constants as parameters):
+``value_dim`` (values of another width than keys); ``conv_taps`` (a short causal
+convolution over time on every channel of q, k and v, straight after the projection:
+``y_t = sum_j c[:, j] * u_(t - taps + 1 + j)``, the last taps - 1 projected rows of a request kept
+as fixed-size state); ``unit_norm_eps`` (after the rotation, q and k heads are divided by their
+root mean square, no weight); ``chunk`` (token i sees key j <= i only if both lie in the same
+run of ``chunk`` positions counted from position 0); ``sink`` (a learned number per query head
+whose exponential joins the softmax's denominator, without key or value); ``output_gate``
+(the concatenated heads times sigmoid(W_g x) before the output projection); ``names`` (what the
+tensors are called in the checkpoint).  With any of them the step takes the general path:
+one product for q, k, v (and the gate), one kernel for convolution, rotation, norms and the
+page write, the masked attention kernel, the gate, the output projection.
 """
 
 from __future__ import annotations
@@ -14,7 +27,7 @@ from __future__ import annotations
 import torch
 from torch import Tensor
 
-from ..cache.spec import CacheNeeds, CacheView, PagedKV
+from ..cache.spec import CacheNeeds, CacheView, FixedState, PagedKV
 from ..kernels import ops
 from ..registry import register_part
 from .base import BuildContext, Mixer, ParamSpec, build_part
@@ -24,7 +37,10 @@ from .plan import PartSpec
 class GroupedQueryAttention(Mixer):
     def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, num_heads: int,
                  num_kv_heads: int, head_dim: int, position: PartSpec, qk_norm_eps: float | None = None,
-                 bias: bool = False, window: int | None = None, scale: float | None = None) -> None:
+                 bias: bool = False, window: int | None = None, scale: float | None = None,
+                 value_dim: int | None = None, conv_taps: int = 0, unit_norm_eps: float | None = None,
+                 chunk: int | None = None, sink: bool = False, output_gate: bool = False,
+                 names: dict[str, str] | None = None) -> None:
         super().__init__(ctx, prefix)
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
@@ -34,17 +50,40 @@ class GroupedQueryAttention(Mixer):
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
         self.head_dim = head_dim
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
         self.q_size = num_heads * head_dim
         self.kv_size = num_kv_heads * head_dim
+        self.v_size = num_kv_heads * self.value_dim
+        self.out_size = num_heads * self.value_dim
+        self.conv_taps = int(conv_taps)
+        self.unit_norm_eps = unit_norm_eps
+        self.chunk = chunk
+        self.sink = sink
+        self.output_gate = output_gate
+        if self.conv_taps == 1 or self.conv_taps < 0:
+            raise ValueError("a short convolution has at least two taps (0: none)")
+        if chunk is not None and (chunk < 1 or window is not None):
+            raise ValueError("chunk must be positive and cannot be combined with a window")
+        # the general path: anything the fused kernels of the plain arrangement do not know
+        self.general = bool(self.value_dim != head_dim or self.conv_taps or unit_norm_eps is not None
+                            or chunk is not None or sink or output_gate)
+        if self.general and qk_norm_eps is not None:
+            raise ValueError("weighted q/k norms before the rotation are not combined with the general path's options")
+        self.names = dict(self.DEFAULT_NAMES, **(names or {}))
         self.qk_norm_eps = qk_norm_eps
         self.bias = bias
         self.window = window
         self.scale = head_dim ** -0.5 if scale is None else float(scale)
         self.position = build_part("position", position, ctx)
-        width = self.q_size + 2 * self.kv_size
-        self._rows = {"q_proj": (0, self.q_size), "k_proj": (self.q_size, self.kv_size),
-                      "v_proj": (self.q_size + self.kv_size, self.kv_size)}
+        self.conv_channels = self.q_size + self.kv_size + self.v_size
+        width = self.conv_channels + (self.out_size if output_gate else 0)
+        self._rows = {"q": (0, self.q_size), "k": (self.q_size, self.kv_size),
+                      "v": (self.q_size + self.kv_size, self.v_size)}
+        if output_gate:
+            self._rows["gate"] = (self.conv_channels, self.out_size)
         self._width = width
+        self.conv_weight: Tensor | None = None
+        self.sink_weight: Tensor | None = None
         self.qkv_weight: Tensor | None = None
         self.qkv_bias: Tensor | None = None
         self.o_weight: Tensor | None = None
@@ -53,47 +92,72 @@ class GroupedQueryAttention(Mixer):
         self.k_norm: Tensor | None = None
 
     # ------------------------------------------------------------ tensors
+    DEFAULT_NAMES = {
+        "q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+        "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+        "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
+        "q_conv": "q_proj.conv", "k_conv": "k_proj.conv", "v_conv": "v_proj.conv",
+        "sink": "sink", "gate": "gate_proj.weight",
+    }
+
     def param_specs(self):
+        n = {key: self.name(leaf) for key, leaf in self.names.items()}
         specs = {
-            self.name("q_proj.weight"): ParamSpec((self.q_size, self.hidden_size)),
-            self.name("k_proj.weight"): ParamSpec((self.kv_size, self.hidden_size)),
-            self.name("v_proj.weight"): ParamSpec((self.kv_size, self.hidden_size)),
-            self.name("o_proj.weight"): ParamSpec((self.hidden_size, self.q_size)),
+            n["q"]: ParamSpec((self.q_size, self.hidden_size)),
+            n["k"]: ParamSpec((self.kv_size, self.hidden_size)),
+            n["v"]: ParamSpec((self.v_size, self.hidden_size)),
+            n["o"]: ParamSpec((self.hidden_size, self.out_size)),
         }
         if self.bias:
-            specs[self.name("q_proj.bias")] = ParamSpec((self.q_size,), kind="vector", init="zeros")
-            specs[self.name("k_proj.bias")] = ParamSpec((self.kv_size,), kind="vector", init="zeros")
-            specs[self.name("v_proj.bias")] = ParamSpec((self.kv_size,), kind="vector", init="zeros")
-            specs[self.name("o_proj.bias")] = ParamSpec((self.hidden_size,), kind="vector", init="zeros")
+            specs[n["q_bias"]] = ParamSpec((self.q_size,), kind="vector", init="zeros")
+            specs[n["k_bias"]] = ParamSpec((self.kv_size,), kind="vector", init="zeros")
+            specs[n["v_bias"]] = ParamSpec((self.v_size,), kind="vector", init="zeros")
+            specs[n["o_bias"]] = ParamSpec((self.hidden_size,), kind="vector", init="zeros")
         if self.qk_norm_eps is not None:
-            specs[self.name("q_norm.weight")] = ParamSpec((self.head_dim,), kind="vector", init="norm")
-            specs[self.name("k_norm.weight")] = ParamSpec((self.head_dim,), kind="vector", init="norm")
+            specs[n["q_norm"]] = ParamSpec((self.head_dim,), kind="vector", init="norm")
+            specs[n["k_norm"]] = ParamSpec((self.head_dim,), kind="vector", init="norm")
+        if self.conv_taps:
+            specs[n["q_conv"]] = ParamSpec((self.q_size, self.conv_taps), kind="vector", init="taps")
+            specs[n["k_conv"]] = ParamSpec((self.kv_size, self.conv_taps), kind="vector", init="taps")
+            specs[n["v_conv"]] = ParamSpec((self.v_size, self.conv_taps), kind="vector", init="taps")
+        if self.sink:
+            specs[n["sink"]] = ParamSpec((self.num_heads,), kind="vector", init="unit")
+        if self.output_gate:
+            specs[n["gate"]] = ParamSpec((self.out_size, self.hidden_size))
         return specs
 
     def set_param(self, name: str, tensor: Tensor) -> None:
         local = name[len(self.prefix) + 1:] if self.prefix else name
-        module, _, leaf = local.rpartition(".")
-        if module in self._rows:
-            start, size = self._rows[module]
-            if leaf == "weight":
-                if self.qkv_weight is None:  # the three projections share one matrix: one product per step
-                    self.qkv_weight = torch.empty((self._width, self.hidden_size), dtype=tensor.dtype,
-                                                  device=tensor.device)
-                if tensor.dtype != self.qkv_weight.dtype:
-                    raise ValueError(f"{name}: q, k and v projections must be stored in one dtype")
-                self.qkv_weight[start:start + size].copy_(tensor)
-            else:
-                if self.qkv_bias is None:
-                    self.qkv_bias = torch.zeros(self._width, dtype=torch.float32, device=tensor.device)
-                self.qkv_bias[start:start + size].copy_(tensor)
-        elif local == "o_proj.weight":
+        key = next((k for k, leaf in self.names.items() if leaf == local), None)
+        if key in self._rows:
+            start, size = self._rows[key]
+            if self.qkv_weight is None:  # the projections share one matrix: one product per step
+                self.qkv_weight = torch.empty((self._width, self.hidden_size), dtype=tensor.dtype,
+                                              device=tensor.device)
+            if tensor.dtype != self.qkv_weight.dtype:
+                raise ValueError(f"{name}: the projections of one input must be stored in one dtype")
+            self.qkv_weight[start:start + size].copy_(tensor)
+        elif key in ("q_bias", "k_bias", "v_bias"):
+            start, size = self._rows[key[0]]
+            if self.qkv_bias is None:
+                self.qkv_bias = torch.zeros(self._width, dtype=torch.float32, device=tensor.device)
+            self.qkv_bias[start:start + size].copy_(tensor)
+        elif key in ("q_conv", "k_conv", "v_conv"):
+            start, size = self._rows[key[0]]
+            if self.conv_weight is None:
+                self.conv_weight = torch.zeros((self.conv_channels, self.conv_taps), dtype=torch.float32,
+                                               device=tensor.device)
+            self.conv_weight[start:start + size].copy_(tensor)
+        elif key == "o":
             self.o_weight = tensor
-        elif local == "o_proj.bias":
+        elif key == "o_bias":
             self.o_bias = tensor
-        elif local == "q_norm.weight":
+        elif key == "q_norm":
             self.q_norm = tensor
-        elif local == "k_norm.weight":
+        elif key == "k_norm":
             self.k_norm = tensor
+        elif key == "sink":
+            self.sink_weight = tensor
         else:
             raise KeyError(name)
 
@@ -105,11 +169,19 @@ class GroupedQueryAttention(Mixer):
 
     def split_qkv_weight(self) -> dict[str, Tensor]:
         """The three projection matrices back out of the fused one."""
-        return {module: self.qkv_weight[start:start + size] for module, (start, size) in self._rows.items()}
+        named = {"q": "q_proj", "k": "k_proj", "v": "v_proj"}
+        return {named[key]: self.qkv_weight[start:start + size] for key, (start, size) in self._rows.items() if key in named}
 
     # ------------------------------------------------------------ running
     def cache_needs(self) -> CacheNeeds:
-        return CacheNeeds(paged=PagedKV(self.num_kv_heads, self.head_dim, self.window))
+        paged = PagedKV(self.num_kv_heads, self.head_dim, self.window,
+                        None if self.value_dim == self.head_dim else self.value_dim, chunk=self.chunk)
+        if not self.conv_taps:
+            return CacheNeeds(paged=paged)
+        # the last taps - 1 projected rows (q, k and v channels), exact in float32
+        return CacheNeeds(paged=paged, state={self.CONV_STATE: FixedState((self.conv_taps - 1, self.conv_channels), torch.float32)})
+
+    CONV_STATE = "conv"
 
     takes_stream = True
 
@@ -117,6 +189,8 @@ class GroupedQueryAttention(Mixer):
                 stream: Tensor | None = None) -> Tensor | None:
         rotary = self.position.rotary()
         inv_freq, rotary_dim = rotary if rotary is not None else (None, 0)
+        if self.general:
+            return self._forward_general(x, batch, cache, writes_cache, stream, inv_freq, rotary_dim)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 1.0
         if writes_cache:
             if self._single_tokens_only(batch, x, cache, rotary_dim):
@@ -149,6 +223,27 @@ class GroupedQueryAttention(Mixer):
             num_decode=batch.num_decode, max_ctx=batch.max_ctx)
         return ops.linear_update(attn, self.o_weight, self.o_bias, stream)   # float32 update for the residual sum
 
+    def _forward_general(self, x: Tensor, batch, cache: CacheView, writes_cache: bool, stream, inv_freq,
+                         rotary_dim: int) -> Tensor | None:
+        if not writes_cache:
+            raise ValueError("the general attention path writes its own keys and values")
+        qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)        # [T, q | k | v (| gate)]
+        q = torch.empty((x.shape[0], self.q_size), dtype=x.dtype, device=x.device)
+        ops.conv_rope_norm_write(
+            qkv, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps else None, inv_freq,
+            batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
+            cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
+            kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,
+            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps, taps=self.conv_taps)
+        attn = torch.empty((x.shape[0], self.out_size), dtype=x.dtype, device=x.device)
+        ops.masked_attention(
+            q, cache.key_pages, cache.value_pages, attn, batch.cu_q, batch.ctx_len, cache.block_table,
+            num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
+            kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim, scale=self.scale,
+            window=self.window, chunk=self.chunk, sink=self.sink_weight,
+            gate=qkv[:, self.conv_channels:] if self.output_gate else None)
+        return ops.linear_update(attn, self.o_weight, self.o_bias, stream)
+
     def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
         """Every sequence of the step brings one token, and the sizes are ones that the
         decode kernel prepares queries and keys for itself."""
@@ -161,6 +256,8 @@ class GroupedQueryAttention(Mixer):
         return self.position.token_inputs()
 
     def kernel_libraries(self):
+        if self.general:
+            return {"conv_rope", "attention_masked", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
         return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 
 

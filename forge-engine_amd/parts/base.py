@@ -32,7 +32,8 @@ class ParamSpec:
     kind: ``matrix`` (kept in the compute dtype), ``vector`` (norm weights and
     biases, widened to float32, which is exact), ``int_table`` (int32).
     ``init``: how the random-weights mode draws it: ``normal`` N(0, 0.02),
-    ``norm`` 1 + N(0, 0.05), ``zeros``.
+    ``norm`` 1 + N(0, 0.05), ``zeros``, ``unit`` N(0, 0.25), ``uniform`` U(0, 1), ``taps`` (a short
+    convolution: N(0, 0.04) with one added to the newest tap).
     """
 
     shape: tuple[int, ...]
@@ -82,6 +83,10 @@ class Part:
         self.prefix = prefix
 
     def name(self, local: str) -> str:
+        """The checkpoint name of one of this part's tensors; an empty ``local`` is the prefix
+        itself (a design that names a part's only tensor like the part)."""
+        if not local:
+            return self.prefix
         return f"{self.prefix}.{local}" if self.prefix else local
 
     def param_specs(self) -> dict[str, ParamSpec]:
@@ -165,15 +170,26 @@ class Head(Part):
 class Block(Part):
     role = "block"
 
-    def __init__(self, ctx: BuildContext, mixer: Mixer, feed_forward: FeedForward,
-                 norms: dict[str, Norm]) -> None:
-        super().__init__(ctx)
+    def __init__(self, ctx: BuildContext, mixer: Mixer, feed_forward: FeedForward | None,
+                 norms: dict[str, Norm], prefix: str = "") -> None:
+        """``feed_forward`` None: a layer without one.  ``prefix``: where tensors of the
+        arrangement itself live (most arrangements have none)."""
+        super().__init__(ctx, prefix)
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norms = norms
 
     def children(self) -> list[Part]:
-        return [self.mixer, self.feed_forward, *self.norms.values()]
+        """The arrangement itself (it may own tensors) and the parts it arranges."""
+        found: list[Part] = [self, self.mixer]
+        if self.feed_forward is not None:
+            found.append(self.feed_forward)
+        return [*found, *self.norms.values()]
+
+    def cache_needs(self) -> CacheNeeds:
+        """What one call of the layer asks of the cache: the mixer's needs, and whatever
+        fixed-size state the arrangement keeps itself (by names that the mixer does not use)."""
+        return self.mixer.cache_needs()
 
     def forward(self, residual: Residual, batch, cache: CacheView | None, writes_cache: bool = True) -> None:
         raise NotImplementedError

@@ -2,9 +2,15 @@
 
 from __future__ import annotations
 
-from ..cache.spec import CacheView
+import dataclasses
+
+import torch
+from torch import Tensor
+
+from ..cache.spec import CacheNeeds, CacheView, FixedState
+from ..kernels import ops
 from ..registry import register_part
-from .base import Block, Residual
+from .base import Block, BuildContext, ParamSpec, Residual
 
 
 class PreNormBlock(Block):
@@ -27,4 +33,64 @@ class PreNormBlock(Block):
             residual.add(self.feed_forward.forward(y, batch))
 
 
+class OutputNormBlock(Block):
+    """Norms on the sublayers' outputs only: ``h += norm_m(mixer(s)); h += norm_f(ffn(h))``.
+    The sublayers read the stream itself.  With ``token_shift`` the mixer reads
+    ``s_t = h_t + (h_(t-1) - h_t) * shift`` instead of ``h_t`` (element by element, h_(-1) = 0),
+    where ``shift`` is a learned vector of the layer; the last h of every request is kept as
+    fixed-size state, so a request may be cut into steps anywhere.  A layer may have no
+    feed-forward."""
+
+    NORMS = ("mixer_out", "ff_out")
+    SHIFT_STATE = "block.shift"
+
+    def __init__(self, ctx: BuildContext, mixer, feed_forward, norms, prefix: str = "", *,
+                 hidden_size: int, token_shift: bool = False, shift_leaf: str = "shift") -> None:
+        super().__init__(ctx, mixer, feed_forward, norms, prefix)
+        self.hidden_size = hidden_size
+        self.token_shift = token_shift
+        self.shift_leaf = shift_leaf
+        self.shift: Tensor | None = None
+
+    def param_specs(self):
+        if not self.token_shift:
+            return {}
+        return {self.name(self.shift_leaf): ParamSpec((self.hidden_size,), kind="vector", init="uniform")}
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        if not self.token_shift or name != self.name(self.shift_leaf):
+            raise KeyError(name)
+        self.shift = tensor.reshape(1, self.hidden_size).contiguous()
+
+    def cache_needs(self) -> CacheNeeds:
+        needs = self.mixer.cache_needs()
+        if not self.token_shift:
+            return needs
+        states = needs.states()
+        if self.SHIFT_STATE in states:
+            raise ValueError(f"the mixer's state '{self.SHIFT_STATE}' collides with the layer's own")
+        states[self.SHIFT_STATE] = FixedState((self.hidden_size,), torch.float32)
+        return CacheNeeds(paged=needs.paged, state=states)
+
+    def forward(self, residual: Residual, batch, cache: CacheView | None, writes_cache: bool = True) -> None:
+        h = residual.flush()
+        if self.token_shift:
+            s = ops.token_shift(h, self.shift, cache.states[self.SHIFT_STATE], batch.cu_q, batch.token_seq,
+                                batch.state_slots, num_seqs=batch.num_seqs, out_dtype=self.ctx.dtype)[0]
+            mixer_cache = dataclasses.replace(
+                cache, states={n: t for n, t in cache.states.items() if n != self.SHIFT_STATE})
+        else:
+            s = ops.cast_rows(h, self.ctx.dtype)
+            mixer_cache = cache
+        residual.add(self.mixer.forward(s, batch, mixer_cache, writes_cache))
+        x = self.norms["mixer_out"].forward(residual)
+        if self.feed_forward is not None:
+            residual.add(self.feed_forward.forward(x, batch))
+            self.norms["ff_out"].forward(residual)
+
+    def kernel_libraries(self):
+        return {"stream_ops"}
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "output_norm", OutputNormBlock)

@@ -17,17 +17,19 @@ from .base import BuildContext, Embedding, Head, ParamSpec, Residual
 
 
 class TokenEmbedding(Embedding):
-    def __init__(self, ctx: BuildContext, prefix: str, *, vocab_size: int, hidden_size: int) -> None:
+    def __init__(self, ctx: BuildContext, prefix: str, *, vocab_size: int, hidden_size: int,
+                 leaf: str = "weight") -> None:
         super().__init__(ctx, prefix)
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.leaf = leaf        # the table's name behind the prefix ("": the prefix itself)
         self.weight: Tensor | None = None
 
     def param_specs(self):
-        return {self.name("weight"): ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.name(self.leaf): ParamSpec((self.vocab_size, self.hidden_size))}
 
     def set_param(self, name: str, tensor: Tensor) -> None:
-        if name != self.name("weight"):
+        if name != self.name(self.leaf):
             raise KeyError(name)
         self.weight = tensor
 
@@ -42,11 +44,12 @@ class TokenEmbedding(Embedding):
 
 class LMHead(Head):
     def __init__(self, ctx: BuildContext, prefix: str, *, vocab_size: int, hidden_size: int,
-                 tied: bool = False) -> None:
+                 tied: bool = False, leaf: str = "weight") -> None:
         super().__init__(ctx, prefix)
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied = tied
+        self.leaf = leaf
         self.weight: Tensor | None = None
         self._embedding: TokenEmbedding | None = None
 
@@ -56,10 +59,10 @@ class LMHead(Head):
     def param_specs(self):
         if self.tied:
             return {}
-        return {self.name("weight"): ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.name(self.leaf): ParamSpec((self.vocab_size, self.hidden_size))}
 
     def set_param(self, name: str, tensor: Tensor) -> None:
-        if self.tied or name != self.name("weight"):
+        if self.tied or name != self.name(self.leaf):
             raise KeyError(name)
         self.weight = tensor
 

@@ -53,4 +53,49 @@ class SwiGLU(FeedForward):
         return {"rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile"}
 
 
+class PolyNormMLP(FeedForward):
+    """``down(act(up(x)))`` with the PolyNorm activation: ``a N(z) + b N(z^2) + c N(z^3) + e``, powers
+    element by element, N dividing a token's vector by its root mean square (float32, epsilon
+    inside the root); the four numbers a, b, c, e are a tensor of the layer."""
+
+    def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, intermediate_size: int, eps: float,
+                 names: dict[str, str] | None = None) -> None:
+        super().__init__(ctx, prefix)
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.eps = float(eps)
+        self.names = dict({"up": "up", "down": "down", "act": "act"}, **(names or {}))
+        self.up_weight: Tensor | None = None
+        self.down_weight: Tensor | None = None
+        self.coefficients: Tensor | None = None
+
+    def param_specs(self):
+        inter, hidden = self.intermediate_size, self.hidden_size
+        return {
+            self.name(self.names["up"]): ParamSpec((inter, hidden)),
+            self.name(self.names["down"]): ParamSpec((hidden, inter)),
+            self.name(self.names["act"]): ParamSpec((4,), kind="vector", init="unit"),
+        }
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        if name == self.name(self.names["up"]):
+            self.up_weight = tensor
+        elif name == self.name(self.names["down"]):
+            self.down_weight = tensor
+        elif name == self.name(self.names["act"]):
+            self.coefficients = tensor
+        else:
+            raise KeyError(name)
+
+    def forward(self, x: Tensor, batch=None) -> Tensor:
+        z = ops.linear(x, self.up_weight)
+        act = torch.empty_like(z)
+        ops.polynorm(z, self.coefficients, self.eps, act)
+        return ops.linear_update(act, self.down_weight)
+
+    def kernel_libraries(self):
+        return {"stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "polynorm_mlp", PolyNormMLP)

@@ -26,8 +26,10 @@ class LayerSpec:
 
     block: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None     # None: the layer has no feed-forward
     norms: dict[str, PartSpec]
+    block_params: dict[str, Any] = field(default_factory=dict)   # constants of the arrangement itself
+    prefix: str = ""                                             # where the arrangement's own tensors live
 
 
 @dataclass(frozen=True)

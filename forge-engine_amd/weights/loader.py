@@ -71,6 +71,19 @@ def checkpoint_files(folder: Path) -> dict[str, Path]:
     return names
 
 
+def checkpoint_shapes(folder: Path) -> dict[str, tuple[int, ...]]:
+    """Tensor name -> shape, from the files' headers alone."""
+    by_file: dict[Path, list[str]] = {}
+    for name, path in checkpoint_files(folder).items():
+        by_file.setdefault(path, []).append(name)
+    shapes = {}
+    for path, names in by_file.items():
+        with safe_open(str(path), framework="pt", device="cpu") as handle:
+            for name in names:
+                shapes[name] = tuple(handle.get_slice(name).get_shape())
+    return shapes
+
+
 def _short(items, limit: int = 12) -> str:
     items = list(items)
     shown = ", ".join(str(item) for item in items[:limit])

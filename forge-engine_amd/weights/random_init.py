@@ -30,6 +30,14 @@ def _draw(spec: ParamSpec, generator: torch.Generator, device) -> torch.Tensor:
     noise = torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device)
     if spec.init == "norm":
         return 1.0 + noise * NORM_STD
+    if spec.init == "unit":        # learned scalars and offsets of order one (sinks, bonuses, decay offsets)
+        return noise * 0.5
+    if spec.init == "uniform":     # blend weights between a token and the one before it
+        return torch.rand(spec.shape, generator=generator, dtype=torch.float32, device=device)
+    if spec.init == "taps":        # short convolutions: most weight on the newest tap, so signals pass
+        taps = noise * 0.2
+        taps[..., -1] += 1.0
+        return taps
     return noise * MATRIX_STD
 
 

@@ -280,6 +280,217 @@ def sample_filtered_rows(logits, params, tokens, status, any_top_k=True, any_top
         tokens[r] = min(pick, logits.shape[1] - 1)
 
 
+# ------------------------------------------------- ops on the stream, beside the matrix products
+
+def cast_rows(h, dtype):
+    return h if h.dtype == dtype else h.to(dtype)
+
+
+def _sum_parts(update):
+    return update.float().sum(0) if update.dim() == 3 else update.float()
+
+
+def _unit(x, eps):
+    return x * torch.rsqrt(x.square().mean(-1, keepdim=True) + eps)
+
+
+def token_shift(x, weights, state, cu_q, token_seq, state_slots, *, num_seqs, out_dtype):
+    xf = x.float()
+    previous = torch.zeros_like(xf)
+    for s in range(num_seqs):
+        a, b = int(cu_q[s]), int(cu_q[s + 1])
+        if b > a:
+            previous[a] = state[int(state_slots[s])]
+            previous[a + 1:b] = xf[a:b - 1]
+    out = (xf[None] + (previous - xf)[None] * weights[:, None, :]).to(out_dtype)
+    for s in range(num_seqs):
+        a, b = int(cu_q[s]), int(cu_q[s + 1])
+        if b > a:
+            state[int(state_slots[s])] = xf[b - 1]
+    return out
+
+
+def rmsnorm_update(h, update, weight, eps, out=None):
+    h += _unit(_sum_parts(update), eps) * weight
+    if out is not None:
+        out.copy_(h.to(out.dtype))
+    return out
+
+
+def rmsnorm_mean(updates, weights, eps, out):
+    total = torch.zeros_like(out)
+    for index, update in enumerate(updates):
+        total += _unit(_sum_parts(update), eps) * weights[index]
+    out.copy_(total / len(updates))
+    return out
+
+
+def polynorm(z, coefficients, eps, out):
+    y = z.float()
+    a, b, c, e = (float(v) for v in coefficients)
+    out.copy_((a * _unit(y, eps) + b * _unit(y * y, eps) + c * _unit(y * y * y, eps) + e).to(out.dtype))
+    return out
+
+
+def tanh_rows(x):
+    x.copy_(torch.tanh(x.float()).to(x.dtype))
+    return x
+
+
+def _act(gate, act):
+    if act == "silu":
+        return gate * torch.sigmoid(gate)
+    if act == "sigmoid":
+        return torch.sigmoid(gate)
+    return torch.ones_like(gate)
+
+
+def head_norm_gate(o, weight, gate, out, *, heads, dim, eps, act="none", extra=0, floor=None):
+    tokens = o.shape[0]
+    y = o[..., :dim]
+    if extra:
+        y = y / (torch.maximum(o[..., dim].abs(), floor) + 1e-6)[..., None]
+    y = _unit(y, eps)
+    if weight is not None:
+        y = y * (weight.view(heads, dim) if weight.numel() == heads * dim else weight.view(1, dim))
+    y = y.reshape(tokens, heads * dim)
+    if gate is not None:
+        y = y * _act(gate.float(), act)
+    out.copy_(y.to(out.dtype))
+    return out
+
+
+def conv_rope_norm_write(qkv, conv_weight, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, block_table,
+                         key_pages, value_pages, q_out, *, num_seqs, q_heads, kv_heads, head_dim, value_dim, rotary_dim,
+                         unit_norm_eps, taps):
+    tokens = qkv.shape[0]
+    q_size, k_size, v_size = q_heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
+    channels = q_size + k_size + v_size
+    u = qkv[:, :channels].float()
+    y = u.clone()
+    if taps:
+        for s in range(num_seqs):
+            a, b = int(cu_q[s]), int(cu_q[s + 1])
+            if b == a:
+                continue
+            slot = int(state_slots[s])
+            history = torch.cat([conv_state[slot], u[a:b]])            # [taps - 1 + n, channels]
+            y[a:b] = sum(history[j:j + b - a] * conv_weight[:, j] for j in range(taps))
+            conv_state[slot] = history[-(taps - 1):]
+
+    def rotate_norm(x):
+        if rotary_dim:
+            half = rotary_dim // 2
+            angle = positions.float().view(-1, 1, 1) * inv_freq.view(1, 1, half)
+            cos, sin = angle.cos(), angle.sin()
+            lo, hi = x[..., :half], x[..., half:rotary_dim]
+            x = torch.cat((lo * cos - hi * sin, hi * cos + lo * sin, x[..., rotary_dim:]), dim=-1)
+        if unit_norm_eps is not None:
+            x = _unit(x, unit_norm_eps)
+        return x
+
+    q = rotate_norm(y[:, :q_size].view(tokens, q_heads, head_dim))
+    k = rotate_norm(y[:, q_size:q_size + k_size].view(tokens, kv_heads, head_dim)).to(qkv.dtype)
+    v = y[:, q_size + k_size:].view(tokens, kv_heads, value_dim).to(qkv.dtype)
+    q_out.copy_(q.reshape(tokens, q_size).to(q_out.dtype))
+    block_size = key_pages.shape[2]
+    for t in range(tokens):
+        pos = int(positions[t])
+        page = int(block_table[int(token_seq[t]), pos // block_size])
+        assert page >= 0, "token without a page"
+        key_pages[page, :, pos % block_size] = k[t]
+        value_pages[page, :, :, pos % block_size] = v[t]
+
+
+def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, q_heads, kv_heads,
+                     head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None):
+    block_size = key_pages.shape[2]
+    groups = q_heads // kv_heads
+    for s in range(num_seqs):
+        a, b = int(cu_q[s]), int(cu_q[s + 1])
+        ctx = int(ctx_len[s])
+        if b == a:
+            continue
+        keys = gather_pages(key_pages, block_table[s], ctx, block_size)                         # [kv, ctx, D]
+        values = gather_pages(value_pages.transpose(2, 3), block_table[s], ctx, block_size)     # [kv, ctx, Dv]
+        for i in range(b - a):
+            p = ctx - (b - a) + i
+            first = 0
+            if window is not None:
+                first = max(first, p - window + 1)
+            if chunk is not None:
+                first = max(first, p // chunk * chunk)
+            for h in range(q_heads):
+                g = h // groups
+                qv = q[a + i, h * head_dim:(h + 1) * head_dim].float()
+                scores = (keys[g, first:p + 1] @ qv) * scale
+                top = scores.max()
+                if sink is not None:
+                    top = torch.maximum(top, sink[h])
+                e = torch.exp(scores - top)
+                denom = e.sum() + (torch.exp(sink[h] - top) if sink is not None else 0.0)
+                o = (e / denom) @ values[g, first:p + 1]
+                if gate is not None:
+                    o = o * torch.sigmoid(gate[a + i, h * value_dim:(h + 1) * value_dim].float())
+                out[a + i, h * value_dim:(h + 1) * value_dim] = o.to(out.dtype)
+    return out
+
+
+def linear_recurrence(q, k, v, out, state, cu_q, state_slots, *, num_seqs, max_q_len, heads, key_dim, value_dim,
+                      decay=None, decay_kind="none", decay_bias=None, tau=1.0, head_decay=None, in_scale=None,
+                      q_scale=1.0, bonus=None, ones_column=False):
+    tokens = q.shape[0]
+    qf = q.float().reshape(tokens, heads, key_dim) * q_scale
+    kf = k.float().reshape(tokens, heads, key_dim)
+    vf = v.float().reshape(tokens, heads, value_dim)
+    if ones_column:
+        vf = torch.cat([vf, torch.ones(tokens, heads, 1)], dim=-1)
+    a = torch.ones(tokens, heads, key_dim)
+    if decay_kind == "exp_neg_exp":
+        a = torch.exp(-torch.exp(decay + decay_bias)).view(tokens, heads, key_dim)
+    elif decay_kind == "sigmoid_root":
+        a = torch.exp(torch.nn.functional.logsigmoid(decay + decay_bias) / tau).view(tokens, heads, key_dim)
+    if head_decay is not None:
+        a = a * head_decay[..., None]
+    b = torch.ones(tokens, heads) if in_scale is None else in_scale
+    u = None if bonus is None else bonus.reshape(heads, key_dim)
+    for s in range(num_seqs):
+        first, last = int(cu_q[s]), int(cu_q[s + 1])
+        if last == first:
+            continue
+        slot = int(state_slots[s])
+        S = state[slot].transpose(1, 2).clone()               # [heads, key, value]
+        for t in range(first, last):
+            kv = b[t][:, None, None] * kf[t][:, :, None] * vf[t][:, None, :]
+            if u is not None:
+                out[t] = torch.einsum("hkv,hk->hv", S + u[:, :, None] * kv, qf[t])
+                S = a[t][:, :, None] * S + kv
+            else:
+                S = a[t][:, :, None] * S + kv
+                out[t] = torch.einsum("hkv,hk->hv", S, qf[t])
+        state[slot] = S.transpose(1, 2)
+    return out
+
+
+def mlstm_gate_scan(gates, bias, cap, maximum, cu_q, state_slots, out, *, num_seqs, heads):
+    g = gates + bias
+    gi = cap * torch.tanh(g[:, :heads] / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(g[:, heads:] / cap))
+    for s in range(num_seqs):
+        first, last = int(cu_q[s]), int(cu_q[s + 1])
+        if last == first:
+            continue
+        m = maximum[int(state_slots[s])].clone()
+        for t in range(first, last):
+            m_new = torch.maximum(gf[t] + m, gi[t])
+            out[0, t] = torch.exp(gf[t] + m - m_new)
+            out[1, t] = torch.exp(gi[t] - m_new)
+            out[2, t] = torch.exp(-m_new)
+            m = m_new
+        maximum[int(state_slots[s])] = m
+    return out
+
+
 def decode_prepare_supported(*args, **kwargs):
     return False        # on the CPU a step of single tokens takes the two references below in turn
 
@@ -294,7 +505,9 @@ DECODE_SPLITS_TESTED = tuple(range(1, 65))
 
 
 NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
-         "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_filtered_rows")
+         "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_filtered_rows",
+         "cast_rows", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
+         "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan")
 
 
 def install(monkeypatch):
