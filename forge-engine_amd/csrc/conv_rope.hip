@@ -1,0 +1,164 @@
+// From the fused q/k/v projection to queries and cached keys and values, for attention whose
+// projections pass a short causal convolution over time:
+//   y_t[c] = sum_j w[c][j] * u_(t - taps + 1 + j)[c]        (rows before the sequence's start: zeros)
+// then q and k heads are rotated (first rotary_dim dims, dim i pairs with i + rotary_dim / 2,
+// angle = position * inv_freq[i]) and, if asked, divided by their root mean square (no weight);
+// q goes to its own buffer, k and v into their pages (values transposed: [dim][slot]).
+// Rows of a sequence that earlier steps brought come from the sequence's state slot, which holds
+// its last taps - 1 projected rows; a second kernel moves the state on after the first has read it.
+// One block per token; everything between the loads and the stores is float32.
+#include "common.h"
+
+#define CR_THREADS 256
+
+template <typename T>
+__global__ __launch_bounds__(CR_THREADS) void conv_rope_norm_write_kernel(
+    const T* __restrict__ qkv, size_t qkv_stride, const float* __restrict__ conv_w,
+    const float* __restrict__ conv_state, const float* __restrict__ inv_freq,
+    const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slots, const int* __restrict__ block_table, int table_stride,
+    T* __restrict__ key_pages, T* __restrict__ value_pages, T* __restrict__ q_out, int q_heads, int kv_heads,
+    int head_dim, int value_dim, int rotary_dim, float eps, int unit_norm, int taps, int block_size,
+    int num_blocks, int slots) {
+  extern __shared__ float y[];   // [channels]
+  const int t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int seq = token_seq[t];
+  const int begin = cu_q[seq];
+  const int pos = positions[t];
+  const int q_size = q_heads * head_dim, k_size = kv_heads * head_dim, v_size = kv_heads * value_dim;
+  const int channels = q_size + k_size + v_size;
+
+  // 1. convolution (or a plain copy) into LDS
+  if (taps > 0) {
+    const int slot = min(max(state_slots[seq], 0), slots - 1);
+    const float* kept = conv_state + (size_t)slot * (taps - 1) * channels;
+    for (int c = tid; c < channels; c += CR_THREADS) {
+      float acc = 0.f;
+      for (int j = 0; j < taps; ++j) {
+        const int row = t - (taps - 1) + j;          // a row of this step, or of the state if before `begin`
+        const float u = row >= begin ? load_as_float(qkv + (size_t)row * qkv_stride + c)
+                                     : kept[(size_t)(taps - 1 - (begin - row)) * channels + c];
+        acc = fmaf(conv_w[(size_t)c * taps + j], u, acc);
+      }
+      y[c] = acc;
+    }
+  } else {
+    for (int c = tid; c < channels; c += CR_THREADS) y[c] = load_as_float(qkv + (size_t)t * qkv_stride + c);
+  }
+  __syncthreads();
+
+  // 2. rotation of q and k heads, a pair per thread
+  const int half = rotary_dim / 2;
+  const int rot_heads = q_heads + kv_heads;
+  for (int e = tid; e < rot_heads * half; e += CR_THREADS) {
+    const int head = e / half, i = e - head * half;
+    float sn, cs;
+    sincosf((float)pos * inv_freq[i], &sn, &cs);
+    float* hv = y + head * head_dim;
+    const float a = hv[i], b = hv[i + half];
+    hv[i] = a * cs - b * sn;
+    hv[i + half] = b * cs + a * sn;
+  }
+  __syncthreads();
+
+  // 3. unit norm per head and the stores: a wave per head
+  const int lane = tid & 63, wave = tid >> 6;
+  const int page = block_table[(size_t)seq * table_stride + pos / block_size];
+  const int place = pos % block_size;
+  const bool paged = page >= 0 && page < num_blocks;
+  for (int head = wave; head < rot_heads; head += CR_THREADS / 64) {
+    const float* hv = y + head * head_dim;
+    float inv = 1.f;
+    if (unit_norm) {
+      float ss = 0.f;
+      for (int c = lane; c < head_dim; c += 64) ss += hv[c] * hv[c];
+      ss = wave_sum(ss);
+      inv = rsqrtf(ss / (float)head_dim + eps);
+    }
+    if (head < q_heads) {
+      T* dst = q_out + (size_t)t * q_size + head * head_dim;
+      for (int c = lane; c < head_dim; c += 64) store_from_float(dst + c, hv[c] * inv);
+    } else if (paged) {
+      T* dst = key_pages + (((size_t)page * kv_heads + (head - q_heads)) * block_size + place) * head_dim;
+      for (int c = lane; c < head_dim; c += 64) store_from_float(dst + c, hv[c] * inv);
+    }
+  }
+  if (paged) {
+    const float* vv = y + q_size + k_size;
+    for (int e = tid; e < v_size; e += CR_THREADS) {
+      const int head = e / value_dim, d = e - head * value_dim;
+      store_from_float(value_pages + (((size_t)page * kv_heads + head) * value_dim + d) * block_size + place, vv[e]);
+    }
+  }
+}
+
+// The state after the step: the last taps - 1 projected rows of every sequence that brought tokens.
+template <typename T>
+__global__ __launch_bounds__(CR_THREADS) void conv_state_update_kernel(
+    const T* __restrict__ qkv, size_t qkv_stride, float* __restrict__ conv_state, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slots, int channels, int taps, int slots, int tokens) {
+  const int seq = blockIdx.y;
+  const int begin = cu_q[seq], end = cu_q[seq + 1];
+  const int slot = state_slots[seq];
+  const int c = blockIdx.x * CR_THREADS + threadIdx.x;
+  if (end <= begin || end > tokens || slot < 0 || slot >= slots || c >= channels) return;
+  const int n = end - begin;
+  float* kept = conv_state + (size_t)slot * (taps - 1) * channels;
+  float next[7];
+#pragma unroll
+  for (int j = 0; j < 7; ++j) {
+    if (j < taps - 1) {
+      const int r = n - (taps - 1) + j;      // relative to the step's first row
+      next[j] = r >= 0 ? load_as_float(qkv + (size_t)(begin + r) * qkv_stride + c)
+                       : kept[(size_t)(taps - 1 + r) * channels + c];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 7; ++j)
+    if (j < taps - 1) kept[(size_t)j * channels + c] = next[j];
+}
+
+extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv_stride, const float* conv_w,
+                                       const float* conv_state, const float* inv_freq, const int* positions,
+                                       const int* token_seq, const int* cu_q, const int* state_slots,
+                                       const int* block_table, int table_stride, void* key_pages, void* value_pages,
+                                       void* q_out, int tokens, int q_heads, int kv_heads, int head_dim, int value_dim,
+                                       int rotary_dim, float eps, int unit_norm, int taps, int block_size,
+                                       int num_blocks, int slots, hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || value_dim <= 0 || block_size <= 0 || num_blocks <= 0)
+    return FE_BAD_ARGUMENT;
+  if (rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 || (rotary_dim && !inv_freq)) return FE_BAD_ARGUMENT;
+  if (taps < 0 || taps == 1 || taps > 8 || (taps && (!conv_w || !conv_state || slots < 1))) return FE_BAD_ARGUMENT;
+  if (unit_norm && !(eps > 0.f)) return FE_BAD_ARGUMENT;
+  const long long channels = (long long)(q_heads + kv_heads) * head_dim + (long long)kv_heads * value_dim;
+  if (channels > 16000 || qkv_stride < channels) return FE_BAD_ARGUMENT;      // a token's channels live in LDS
+  const size_t lds = (size_t)channels * sizeof(float);
+#define LAUNCH(T)                                                                                              \
+  conv_rope_norm_write_kernel<T><<<tokens, CR_THREADS, lds, stream>>>(                                         \
+      (const T*)qkv, (size_t)qkv_stride, conv_w, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, \
+      block_table, table_stride, (T*)key_pages, (T*)value_pages, (T*)q_out, q_heads, kv_heads, head_dim,       \
+      value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots)
+  if (dtype == FE_F32) LAUNCH(float);
+  else if (dtype == FE_BF16) LAUNCH(bf16_t);
+  else return FE_BAD_ARGUMENT;
+#undef LAUNCH
+  return fe_check_launch();
+}
+
+extern "C" int fe_conv_state_update(const void* qkv, int dtype, long long qkv_stride, float* conv_state,
+                                    const int* cu_q, const int* state_slots, int num_seqs, int channels, int taps,
+                                    int slots, int tokens, hipStream_t stream) {
+  if (num_seqs <= 0 || tokens <= 0) return FE_OK;
+  if (channels <= 0 || taps < 2 || taps > 8 || slots < 1 || qkv_stride < channels) return FE_BAD_ARGUMENT;
+  const dim3 grid((channels + CR_THREADS - 1) / CR_THREADS, num_seqs);
+  if (dtype == FE_F32)
+    conv_state_update_kernel<float><<<grid, CR_THREADS, 0, stream>>>((const float*)qkv, (size_t)qkv_stride, conv_state,
+                                                                     cu_q, state_slots, channels, taps, slots, tokens);
+  else if (dtype == FE_BF16)
+    conv_state_update_kernel<bf16_t><<<grid, CR_THREADS, 0, stream>>>((const bf16_t*)qkv, (size_t)qkv_stride, conv_state,
+                                                                      cu_q, state_slots, channels, taps, slots, tokens);
+  else return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}

@@ -28,7 +28,7 @@ import json
 import sys
 from pathlib import Path
 
-LIVE_REQUESTS = 8  # state slots of the replay pool (a trace holds up to four requests at a time)
+LIVE_REQUESTS = 4  # state slots of the replay pool: a trace holds up to four requests at a time, so slots are used again
 
 
 def build_parser() -> argparse.ArgumentParser:
