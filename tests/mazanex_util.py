@@ -1,0 +1,93 @@
+"""Small Mazanex configurations for the tests (config.json form), model folders with random
+weights, and the plain implementation's logits for them."""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import torch
+from safetensors.torch import load_file
+
+import plain_mazanex as plain
+
+
+def attention(heads, kv_heads, dim, vdim, conv, chunk, rot_dims, base=10000.0, scale=0.25):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv, "mask": {"size": chunk},
+            "rot": {"dims": rot_dims, "base": base}, "scale": scale}
+
+
+def layer(kind, mixer, ff):
+    return {"type": kind, "mixer": mixer, "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+
+
+def config(vocab, width, layers, eps=1e-6):
+    return {"architecture": "Mazanex", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers}
+
+
+PARALLEL_P = {"left": attention(4, 2, 16, 8, 3, 6, 8, base=500.0, scale=0.3), "right": {"heads": 3, "dim": 16, "rank": 5}}
+PARALLEL_Q = {"left": attention(3, 3, 24, 40, 2, 5, 24, scale=0.2), "right": {"heads": 1, "dim": 40, "rank": 3}}
+GLA_P = {"heads": 2, "dim": 8, "vdim": 24, "tau": 4.0, "rank": 5}
+GLA_Q = {"heads": 3, "dim": 20, "vdim": 12, "tau": 9.5, "rank": 2}
+MLSTM_P = {"heads": 3, "dim": 16, "vdim": 16, "gate_cap": 8.0}
+MLSTM_Q = {"heads": 1, "dim": 24, "vdim": 40, "gate_cap": 15.0}
+
+# every mixer, one layer without a feed-forward, sizes that differ from one another everywhere
+MIXED_A = config(96, 48, [layer("parallel", PARALLEL_P, 80), layer("gla", GLA_P, None), layer("mlstm", MLSTM_P, 56)])
+# another order, a group of one (heads = kv_heads), one head, the whole head rotated, a chunk shorter than a page
+MIXED_B = config(130, 40, [layer("mlstm", MLSTM_Q, 72), layer("parallel", PARALLEL_Q, 36), layer("gla", GLA_Q, 64),
+                           layer("parallel", PARALLEL_P, None)], eps=1e-5)
+ALONE = {
+    "parallel": config(64, 32, [layer("parallel", PARALLEL_P, None)]),
+    "gla": config(64, 32, [layer("gla", GLA_Q, None)]),
+    "mlstm": config(64, 32, [layer("mlstm", MLSTM_P, None)]),
+    "feed_forward": config(64, 32, [layer("gla", GLA_P, 50)]),
+}
+BLOCK_SIZE = {"A": 4, "B": 8}
+
+
+def write_model(raw: dict, seed: int, folder) -> Path:
+    from forge_engine_amd.config import load_model_config
+    from forge_engine_amd.weights import write_random_model
+
+    return write_random_model(load_model_config(raw), seed, folder)
+
+
+def folder_weights(folder) -> tuple[dict, dict]:
+    folder = Path(folder)
+    return json.loads((folder / "config.json").read_text()), load_file(str(folder / "model.safetensors"))
+
+
+def plain_logits(folder, requests, only=None) -> dict[tuple[str, int], torch.Tensor]:
+    """(request, position) -> logits row of the plain implementation (float64, returned as float32)."""
+    raw, weights = folder_weights(folder)
+    want = {}
+    for request_id, tokens in requests.items():
+        logits = plain.forward(raw, weights, tokens).float()
+        for position in range(len(tokens)):
+            if only is None or (request_id, position) in only:
+                want[(request_id, position)] = logits[position]
+    return want
+
+
+def plain_greedy(folder, prompt, count) -> list[int]:
+    raw, weights = folder_weights(folder)
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(plain.forward(raw, weights, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+def compare(got: dict, want: dict, dtype: str, fraction: float | None = None) -> float:
+    """Largest difference as a fraction of the logits' spread; the bound is that of float32 sums in
+    another order (recurrences over tens of tokens included), or of bfloat16 activations."""
+    assert set(got) == set(want), "not every wanted row came back"
+    scale = max(float((v - v.mean()).abs().max()) for v in want.values())
+    bound = fraction if fraction is not None else (2e-4 if dtype == "float32" else 0.03)
+    worst = 0.0
+    for key in sorted(want):
+        assert torch.isfinite(got[key]).all(), f"non-finite logits at {key}"
+        diff = float((got[key] - want[key]).abs().max()) / scale
+        assert diff <= bound, f"{dtype} logits differ at {key}: {diff:.3e} of the spread > {bound:.1e}"
+        worst = max(worst, diff)
+    return worst

@@ -133,7 +133,8 @@ def run_trace(model_dir, dtype: str, trace: TraceBuilder, out_dir, *, block_size
                      max_tokens=trace.peak_tokens if max_tokens is None else max_tokens, device=device)
     assert replay.run(args, stdin=stdin, stdout=stdout, device="cpu" if on_cpu else None) == 0
     assert stdout.getvalue().split() == [w for s in trace.steps for w in ("done", str(s["step"]))]
-    return collect(trace, out_dir, json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"])
+    config = json.loads((Path(model_dir) / "config.json").read_text())
+    return collect(trace, out_dir, config["vocab_size"] if "vocab_size" in config else config["vocab"])
 
 
 def collect(trace: TraceBuilder, out_dir, vocab: int):
