@@ -110,7 +110,9 @@ def parse_args():
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     parser.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     parser.add_argument("--points", default=None, help="other decode batch sizes to report")
-    parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro", "check"), default="all",
+    parser.add_argument("--widths", default="1024,2048,4096",
+                        help="--phase design: model widths at which Mazanex and Qwen3 are measured side by side")
+    parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro", "check", "design"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
     parser.add_argument("--through", choices=("step", "scheduler"), default="step",
                         help="decode by calling the step function, or through the scheduler's step()")
@@ -137,11 +139,23 @@ def weight_bytes(model) -> int:
     """Bytes of every tensor a decode step reads once (the embedding matrix
     counts once: as the head of a tied model, or as the head's own matrix)."""
     seen, total = set(), 0
-    for part in model.parts():
-        for value in vars(part).values():
-            if hasattr(value, "data_ptr") and hasattr(value, "element_size") and value.data_ptr() not in seen:
+
+    def walk(value, depth=0):
+        nonlocal total
+        if hasattr(value, "data_ptr") and hasattr(value, "element_size"):
+            if value.data_ptr() not in seen:
                 seen.add(value.data_ptr())
                 total += value.numel() * value.element_size()
+        elif isinstance(value, dict) and depth < 6:          # tensors by name, parts by name (mixers side by side)
+            for inner in value.values():
+                walk(inner, depth + 1)
+        elif hasattr(value, "param_specs") and hasattr(value, "ctx") and depth < 6 and id(value) not in seen:
+            seen.add(id(value))
+            for inner in vars(value).values():
+                walk(inner, depth + 1)
+
+    for part in model.parts():
+        walk(part)
     if not getattr(model.head, "tied", False):
         total -= model.embedding.weight.numel() * model.embedding.weight.element_size()
     return total
@@ -273,6 +287,91 @@ def cross_check(args) -> int:
     return 0
 
 
+def design_configs(width: int, layers: int) -> dict:
+    """Mazanex and Qwen3 at one width with layers of equal size: heads of 128, a group of four, a
+    feed-forward three times the width, the same vocabulary and layer count.  Mazanex cycles through
+    its three mixers (parallel attention + RWKV, gated linear attention, mLSTM)."""
+    heads = max(4, width // 128)
+    attention = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "conv": 4, "mask": {"size": 2048},
+                 "rot": {"dims": 64, "base": 10000.0}, "scale": 128 ** -0.5}
+    mixers = [("parallel", {"left": attention, "right": {"heads": width // 64, "dim": 64, "rank": 64}}),
+              ("gla", {"heads": heads, "dim": 64, "vdim": 128, "tau": 16.0, "rank": 16}),
+              ("mlstm", {"heads": max(2, heads // 2), "dim": 128, "vdim": 256, "gate_cap": 15.0})]
+    mazanex = {"architecture": "Mazanex", "vocab": 32000, "width": width, "norm": {"eps": 1e-6},
+               "layers": [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": {"kind": "dense", "ff": 3 * width}}
+                          for i in range(layers)]}
+    qwen3 = _qwen3(vocab_size=32000, hidden_size=width, intermediate_size=3 * width, num_hidden_layers=layers,
+                   num_attention_heads=heads, num_key_value_heads=heads // 4, rope_theta=1000000.0,
+                   tie_word_embeddings=False, eos_token_id=None)
+    return {"Mazanex": mazanex, "Qwen3": qwen3}
+
+
+def design_comparison(args) -> int:
+    """Prefill and decode throughput of Mazanex beside Qwen3 (the closest existing model) at equal
+    width, layer count, feed-forward size and vocabulary; random weights, one JSON line a model and width."""
+    import torch
+
+    from forge_engine_amd.config import load_model_config
+    from forge_engine_amd.engine import ModelRunner, StepEntry, random_model
+
+    device = torch.device("cuda:0")
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
+    layers = args.layers or 6
+    batch = args.batch or 8
+    prompt_len = args.prompt_len or 1024
+    generator = torch.Generator().manual_seed(args.seed)
+    for width in (int(w) for w in args.widths.split(",")):
+        for label, raw in design_configs(width, layers).items():
+            config = load_model_config(raw)
+            model = random_model(config, args.seed, dtype=dtype, device=device)
+            pages = -(-(max(args.prefill_tokens, prompt_len) + args.steps + args.warmup + 16) // args.block_size)
+            runner = ModelRunner(model, block_size=args.block_size, block_capacity=(batch + 1) * pages,
+                                 num_state_slots=batch + 1, eager_sightings=1)
+            vocab = raw.get("vocab", raw.get("vocab_size"))
+
+            def tokens(n):
+                return torch.randint(0, vocab, (n,), generator=generator).tolist()
+
+            def time_ms(fn, warmup, steps):
+                for _ in range(warmup):
+                    fn()
+                torch.cuda.synchronize()
+                events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+                for begin, end in events:
+                    begin.record()
+                    fn()
+                    end.record()
+                torch.cuda.synchronize()
+                return spread([begin.elapsed_time(end) for begin, end in events])["median"]
+
+            prompt = tokens(args.prefill_tokens)
+
+            def prefill_once():
+                runner.begin("p")
+                runner.step([StepEntry("p", prompt, [len(prompt) - 1])])
+                runner.end("p")
+
+            prefill_ms = time_ms(prefill_once, 2, max(3, min(10, args.steps)))
+            names = [f"d{i}" for i in range(batch)]
+            for name in names:
+                runner.begin(name)
+                runner.step([StepEntry(name, tokens(prompt_len), [])])
+            entries = [StepEntry(name, [1], [0]) for name in names]
+            decode_ms = time_ms(lambda: runner.step(entries), args.warmup, args.steps)
+            print(json.dumps({
+                "phase": "design", "model": label, "width": width, "layers": layers, "dtype": args.dtype,
+                "weight_gb": round(weight_bytes(model) / 1e9, 3),
+                "prefill_tokens": args.prefill_tokens, "prefill_ms": prefill_ms,
+                "prefill_tokens_per_s": round(args.prefill_tokens / prefill_ms * 1e3, 1),
+                "decode_batch": batch, "decode_context": prompt_len, "decode_ms": decode_ms,
+                "decode_tokens_per_s": round(batch / decode_ms * 1e3, 1),
+                "graph_replays": runner.graph_replays,
+            }), flush=True)
+            del runner, model
+            torch.cuda.empty_cache()
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -282,6 +381,8 @@ def main() -> int:
         return micro_benchmarks()
     if args.phase == "check":
         return cross_check(args)
+    if args.phase == "design":
+        return design_comparison(args)
     import torch
 
     from forge_engine_amd.config import SchedulerConfig, load_model_config

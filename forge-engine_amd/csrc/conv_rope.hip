@@ -6,14 +6,16 @@
 // q goes to its own buffer, k and v into their pages (values transposed: [dim][slot]).
 // Rows of a sequence that earlier steps brought come from the sequence's state slot, which holds
 // its last taps - 1 projected rows; a second kernel moves the state on after the first has read it.
-// One block per token; everything between the loads and the stores is float32.
+// The projection's bias (float32, one entry per q, k and v channel, or none) is added here, to the
+// rows as they are loaded, so that the product before this kernel has none; the state holds rows
+// with their bias.  One block per token; everything between the loads and the stores is float32.
 #include "common.h"
 
 #define CR_THREADS 256
 
 template <typename T>
 __global__ __launch_bounds__(CR_THREADS) void conv_rope_norm_write_kernel(
-    const T* __restrict__ qkv, size_t qkv_stride, const float* __restrict__ conv_w,
+    const T* __restrict__ qkv, size_t qkv_stride, const float* __restrict__ bias, const float* __restrict__ conv_w,
     const float* __restrict__ conv_state, const float* __restrict__ inv_freq,
     const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ cu_q,
     const int* __restrict__ state_slots, const int* __restrict__ block_table, int table_stride,
@@ -35,16 +37,18 @@ __global__ __launch_bounds__(CR_THREADS) void conv_rope_norm_write_kernel(
     const float* kept = conv_state + (size_t)slot * (taps - 1) * channels;
     for (int c = tid; c < channels; c += CR_THREADS) {
       float acc = 0.f;
+      const float b = bias ? bias[c] : 0.f;
       for (int j = 0; j < taps; ++j) {
         const int row = t - (taps - 1) + j;          // a row of this step, or of the state if before `begin`
-        const float u = row >= begin ? load_as_float(qkv + (size_t)row * qkv_stride + c)
+        const float u = row >= begin ? load_as_float(qkv + (size_t)row * qkv_stride + c) + b
                                      : kept[(size_t)(taps - 1 - (begin - row)) * channels + c];
         acc = fmaf(conv_w[(size_t)c * taps + j], u, acc);
       }
       y[c] = acc;
     }
   } else {
-    for (int c = tid; c < channels; c += CR_THREADS) y[c] = load_as_float(qkv + (size_t)t * qkv_stride + c);
+    for (int c = tid; c < channels; c += CR_THREADS)
+      y[c] = load_as_float(qkv + (size_t)t * qkv_stride + c) + (bias ? bias[c] : 0.f);
   }
   __syncthreads();
 
@@ -96,8 +100,8 @@ __global__ __launch_bounds__(CR_THREADS) void conv_rope_norm_write_kernel(
 // The state after the step: the last taps - 1 projected rows of every sequence that brought tokens.
 template <typename T>
 __global__ __launch_bounds__(CR_THREADS) void conv_state_update_kernel(
-    const T* __restrict__ qkv, size_t qkv_stride, float* __restrict__ conv_state, const int* __restrict__ cu_q,
-    const int* __restrict__ state_slots, int channels, int taps, int slots, int tokens) {
+    const T* __restrict__ qkv, size_t qkv_stride, const float* __restrict__ bias, float* __restrict__ conv_state,
+    const int* __restrict__ cu_q, const int* __restrict__ state_slots, int channels, int taps, int slots, int tokens) {
   const int seq = blockIdx.y;
   const int begin = cu_q[seq], end = cu_q[seq + 1];
   const int slot = state_slots[seq];
@@ -110,7 +114,7 @@ __global__ __launch_bounds__(CR_THREADS) void conv_state_update_kernel(
   for (int j = 0; j < 7; ++j) {
     if (j < taps - 1) {
       const int r = n - (taps - 1) + j;      // relative to the step's first row
-      next[j] = r >= 0 ? load_as_float(qkv + (size_t)(begin + r) * qkv_stride + c)
+      next[j] = r >= 0 ? load_as_float(qkv + (size_t)(begin + r) * qkv_stride + c) + (bias ? bias[c] : 0.f)
                        : kept[(size_t)(taps - 1 + r) * channels + c];
     }
   }
@@ -119,7 +123,7 @@ __global__ __launch_bounds__(CR_THREADS) void conv_state_update_kernel(
     if (j < taps - 1) kept[(size_t)j * channels + c] = next[j];
 }
 
-extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv_stride, const float* conv_w,
+extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv_stride, const float* bias, const float* conv_w,
                                        const float* conv_state, const float* inv_freq, const int* positions,
                                        const int* token_seq, const int* cu_q, const int* state_slots,
                                        const int* block_table, int table_stride, void* key_pages, void* value_pages,
@@ -137,7 +141,7 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
   const size_t lds = (size_t)channels * sizeof(float);
 #define LAUNCH(T)                                                                                              \
   conv_rope_norm_write_kernel<T><<<tokens, CR_THREADS, lds, stream>>>(                                         \
-      (const T*)qkv, (size_t)qkv_stride, conv_w, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, \
+      (const T*)qkv, (size_t)qkv_stride, bias, conv_w, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, \
       block_table, table_stride, (T*)key_pages, (T*)value_pages, (T*)q_out, q_heads, kv_heads, head_dim,       \
       value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots)
   if (dtype == FE_F32) LAUNCH(float);
@@ -147,17 +151,17 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
   return fe_check_launch();
 }
 
-extern "C" int fe_conv_state_update(const void* qkv, int dtype, long long qkv_stride, float* conv_state,
+extern "C" int fe_conv_state_update(const void* qkv, int dtype, long long qkv_stride, const float* bias, float* conv_state,
                                     const int* cu_q, const int* state_slots, int num_seqs, int channels, int taps,
                                     int slots, int tokens, hipStream_t stream) {
   if (num_seqs <= 0 || tokens <= 0) return FE_OK;
   if (channels <= 0 || taps < 2 || taps > 8 || slots < 1 || qkv_stride < channels) return FE_BAD_ARGUMENT;
   const dim3 grid((channels + CR_THREADS - 1) / CR_THREADS, num_seqs);
   if (dtype == FE_F32)
-    conv_state_update_kernel<float><<<grid, CR_THREADS, 0, stream>>>((const float*)qkv, (size_t)qkv_stride, conv_state,
+    conv_state_update_kernel<float><<<grid, CR_THREADS, 0, stream>>>((const float*)qkv, (size_t)qkv_stride, bias, conv_state,
                                                                      cu_q, state_slots, channels, taps, slots, tokens);
   else if (dtype == FE_BF16)
-    conv_state_update_kernel<bf16_t><<<grid, CR_THREADS, 0, stream>>>((const bf16_t*)qkv, (size_t)qkv_stride, conv_state,
+    conv_state_update_kernel<bf16_t><<<grid, CR_THREADS, 0, stream>>>((const bf16_t*)qkv, (size_t)qkv_stride, bias, conv_state,
                                                                       cu_q, state_slots, channels, taps, slots, tokens);
   else return FE_BAD_ARGUMENT;
   return fe_check_launch();

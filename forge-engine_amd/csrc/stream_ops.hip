@@ -203,6 +203,21 @@ extern "C" int fe_polynorm(const void* z, int dtype, const float* coeff, float e
   return fe_check_launch();
 }
 
+// ---------------------------------------------------------------- bias of an update
+// update[r][c] += bias[c] for the first `rows * width` elements (the first part of an update in parts).
+__global__ void add_bias_kernel(float* __restrict__ update, const float* __restrict__ bias, long long count, int width) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) update[i] += bias[i % width];
+}
+
+extern "C" int fe_add_bias(float* update, const float* bias, int rows, int width, hipStream_t stream) {
+  if (rows <= 0) return FE_OK;
+  if (width <= 0) return FE_BAD_ARGUMENT;
+  const long long count = (long long)rows * width;
+  add_bias_kernel<<<(int)((count + 255) / 256), 256, 0, stream>>>(update, bias, count, width);
+  return fe_check_launch();
+}
+
 // ---------------------------------------------------------------- tanh in place
 template <typename T>
 __global__ void tanh_kernel(T* __restrict__ x, long long count) {

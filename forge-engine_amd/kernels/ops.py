@@ -1082,6 +1082,17 @@ def polynorm(z: Tensor, coefficients: Tensor, eps: float, out: Tensor) -> Tensor
     return out
 
 
+def add_bias(update: Tensor, bias: Tensor) -> Tensor:
+    """update += bias along the rows, for a float32 update [T, W]; of an update in parts
+    [parts, T, W] the first part takes it (the parts are added up by whoever reads them)."""
+    _gpu(update, "update", torch.float32)
+    _gpu(bias, "bias", torch.float32)
+    if update.dim() not in (2, 3) or bias.shape != (update.shape[-1],):
+        raise KernelError(f"update must be [T, W] or [parts, T, W] and bias [W], got {tuple(update.shape)} and {tuple(bias.shape)}")
+    _call("stream_ops", "fe_add_bias", _ptr(update), _ptr(bias), c_int(update.shape[-2]), c_int(update.shape[-1]), _stream())
+    return update
+
+
 def tanh_rows(x: Tensor) -> Tensor:
     """tanh of every element, in place (float32 inside)."""
     _gpu(x, "x")
@@ -1136,13 +1147,14 @@ def head_norm_gate(o: Tensor, weight: Tensor | None, gate: Tensor | None, out: T
 
 # ------------------------------------------------- short convolution, rotation, unit norm, page write
 
-def conv_rope_norm_write(qkv: Tensor, conv_weight: Tensor | None, conv_state: Tensor | None, inv_freq: Tensor | None,
+def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor | None, conv_state: Tensor | None, inv_freq: Tensor | None,
                          positions: Tensor, token_seq: Tensor, cu_q: Tensor, state_slots: Tensor, block_table: Tensor,
                          key_pages: Tensor, value_pages: Tensor, q_out: Tensor, *, num_seqs: int, q_heads: int,
                          kv_heads: int, head_dim: int, value_dim: int, rotary_dim: int, unit_norm_eps: float | None,
                          taps: int) -> None:
     """From the projection's output to queries and cached keys and values in one kernel: a short
-    causal convolution over time on every q, k and v channel (``taps`` > 0: y_t = sum_j c[:, j] *
+    projection's bias (float32 [channels] or None: the product before has none), a short causal
+    convolution over time on every q, k and v channel (``taps`` > 0: y_t = sum_j c[:, j] *
     u_(t - taps + 1 + j), rows before the step from ``conv_state`` [slots, taps - 1, channels],
     which afterwards holds every sequence's last taps - 1 projected rows); rotation of the first
     ``rotary_dim`` dims of q and k heads (dim i pairs with i + rotary_dim / 2); then q and k heads
@@ -1157,6 +1169,10 @@ def conv_rope_norm_write(qkv: Tensor, conv_weight: Tensor | None, conv_state: Te
     _gpu(q_out, "q_out", qkv.dtype)
     if q_out.shape != (tokens, q_heads * head_dim):
         raise KernelError(f"q_out must be [{tokens}, {q_heads * head_dim}]")
+    if bias is not None:
+        _gpu(bias, "bias", torch.float32)
+        if bias.shape != (channels,):
+            raise KernelError(f"bias must be [{channels}]")
     if taps:
         _gpu(conv_weight, "conv_weight", torch.float32)
         _gpu(conv_state, "conv_state", torch.float32)
@@ -1187,7 +1203,7 @@ def conv_rope_norm_write(qkv: Tensor, conv_weight: Tensor | None, conv_state: Te
         raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
     stride = qkv.stride(0) if tokens > 1 else max(qkv.stride(0), qkv.shape[1])
     slots = conv_state.shape[0] if taps else 0
-    _call("conv_rope", "fe_conv_rope_norm_write", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride),
+    _call("conv_rope", "fe_conv_rope_norm_write", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias),
           _ptr(conv_weight if taps else None), _ptr(conv_state if taps else None), _ptr(inv_freq if rotary_dim else None),
           _ptr(positions), _ptr(token_seq), _ptr(cu_q), _ptr(state_slots), _ptr(block_table), c_int(block_table.stride(0)),
           _ptr(key_pages), _ptr(value_pages), _ptr(q_out), c_int(tokens), c_int(q_heads), c_int(kv_heads), c_int(head_dim),
@@ -1195,7 +1211,7 @@ def conv_rope_norm_write(qkv: Tensor, conv_weight: Tensor | None, conv_state: Te
           c_int(1 if unit_norm_eps is not None else 0), c_int(taps), c_int(block_size), c_int(num_blocks), c_int(slots),
           _stream())
     if taps:
-        _call("conv_rope", "fe_conv_state_update", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(conv_state),
+        _call("conv_rope", "fe_conv_state_update", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias), _ptr(conv_state),
               _ptr(cu_q), _ptr(state_slots), c_int(num_seqs), c_int(channels), c_int(taps), c_int(slots), c_int(tokens),
               _stream())
 

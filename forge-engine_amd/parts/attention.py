@@ -162,6 +162,9 @@ class GroupedQueryAttention(Mixer):
             raise KeyError(name)
 
     def finalize(self) -> None:
+        # the general path adds biases in float32 behind the products, which then take the kernels for few rows
+        self.conv_bias = None if self.qkv_bias is None else self.qkv_bias[:self.conv_channels].float().contiguous()
+        self.o_bias_f32 = None if self.o_bias is None else self.o_bias.float().contiguous()
         if self.qkv_bias is not None and self.qkv_weight.dtype != torch.float32:
             self.qkv_bias = self.qkv_bias.to(self.qkv_weight.dtype)
         if self.o_bias is not None and self.o_weight.dtype != torch.float32:
@@ -227,10 +230,10 @@ class GroupedQueryAttention(Mixer):
                          rotary_dim: int) -> Tensor | None:
         if not writes_cache:
             raise ValueError("the general attention path writes its own keys and values")
-        qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)        # [T, q | k | v (| gate)]
+        qkv = ops.linear(x, self.qkv_weight)        # [T, q | k | v (| gate)]; the bias is added by the kernel below
         q = torch.empty((x.shape[0], self.q_size), dtype=x.dtype, device=x.device)
         ops.conv_rope_norm_write(
-            qkv, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps else None, inv_freq,
+            qkv, self.conv_bias, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps else None, inv_freq,
             batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
             cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,
@@ -242,7 +245,8 @@ class GroupedQueryAttention(Mixer):
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim, scale=self.scale,
             window=self.window, chunk=self.chunk, sink=self.sink_weight,
             gate=qkv[:, self.conv_channels:] if self.output_gate else None)
-        return ops.linear_update(attn, self.o_weight, self.o_bias, stream)
+        update = ops.linear_update(attn, self.o_weight)
+        return update if self.o_bias_f32 is None else ops.add_bias(update, self.o_bias_f32)
 
     def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
         """Every sequence of the step brings one token, and the sizes are ones that the

@@ -360,13 +360,23 @@ def head_norm_gate(o, weight, gate, out, *, heads, dim, eps, act="none", extra=0
     return out
 
 
-def conv_rope_norm_write(qkv, conv_weight, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, block_table,
+def add_bias(update, bias):
+    if update.dim() == 3:
+        update[0] += bias
+    else:
+        update += bias
+    return update
+
+
+def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, block_table,
                          key_pages, value_pages, q_out, *, num_seqs, q_heads, kv_heads, head_dim, value_dim, rotary_dim,
                          unit_norm_eps, taps):
     tokens = qkv.shape[0]
     q_size, k_size, v_size = q_heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
     channels = q_size + k_size + v_size
     u = qkv[:, :channels].float()
+    if bias is not None:
+        u = u + bias
     y = u.clone()
     if taps:
         for s in range(num_seqs):
@@ -506,7 +516,7 @@ DECODE_SPLITS_TESTED = tuple(range(1, 65))
 
 NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
          "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_filtered_rows",
-         "cast_rows", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
+         "cast_rows", "add_bias", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
          "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan")
 
 

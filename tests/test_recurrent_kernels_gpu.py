@@ -103,6 +103,9 @@ def test_polynorm(ops, dtype, rows, width):
     want = refs.polynorm(z, coeff, 1e-6, torch.empty_like(z))
     got = ops.polynorm(z.to(DEV), coeff.to(DEV), 1e-6, torch.empty_like(z, device=DEV))
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+    for shape in ((9, 40), (3, 9, 40)):
+        update, row_bias = rand(g, *shape), rand(g, 40)
+        torch.testing.assert_close(ops.add_bias(update.to(DEV), row_bias.to(DEV)).cpu(), refs.add_bias(update.clone(), row_bias))
     x = rand(g, 1000, dtype=dtype, scale=2.0)
     torch.testing.assert_close(ops.tanh_rows(x.to(DEV)).cpu().float(), refs.tanh_rows(x.clone()).float(), **tol(dtype))
 
@@ -160,18 +163,19 @@ def test_conv_rope_norm_write(ops, dtype, sizes):
     channels = (sizes["q_heads"] + sizes["kv_heads"]) * sizes["head_dim"] + sizes["kv_heads"] * sizes["value_dim"]
     wide = rand(g, tokens, channels + 17, dtype=dtype)
     qkv = wide[:, :channels]
+    bias = rand(g, channels) if sizes["value_dim"] != 32 else None
     conv_w = rand(g, channels, taps) if taps else None
     state = rand(g, 6, taps - 1, channels) if taps else None
     inv_freq = (1.0 / 10000.0 ** (torch.arange(0, rotary_dim, 2).float() / rotary_dim)) if rotary_dim else None
     state_ref = None if state is None else state.clone()
     keys_ref, values_ref = keys.clone(), values.clone()
     q_ref = torch.empty(tokens, sizes["q_heads"] * sizes["head_dim"], dtype=dtype)
-    refs.conv_rope_norm_write(qkv, conv_w, state_ref, inv_freq, positions, seq, cu, slots, table, keys_ref, values_ref, q_ref,
+    refs.conv_rope_norm_write(qkv, bias, conv_w, state_ref, inv_freq, positions, seq, cu, slots, table, keys_ref, values_ref, q_ref,
                               num_seqs=len(lengths), rotary_dim=rotary_dim, unit_norm_eps=1e-6, taps=taps, **geometry)
     wide_d, conv_d, state_d, freq_d, pos_d, seq_d, cu_d, slots_d, table_d, keys_d, values_d = dev(
         wide, conv_w, state, inv_freq, positions, seq, cu, slots, table, keys, values)
     q_d = torch.empty_like(q_ref, device=DEV)
-    ops.conv_rope_norm_write(wide_d[:, :channels], conv_d, state_d, freq_d, pos_d, seq_d, cu_d, slots_d, table_d, keys_d,
+    ops.conv_rope_norm_write(wide_d[:, :channels], None if bias is None else bias.to(DEV), conv_d, state_d, freq_d, pos_d, seq_d, cu_d, slots_d, table_d, keys_d,
                              values_d, q_d, num_seqs=len(lengths), rotary_dim=rotary_dim, unit_norm_eps=1e-6, taps=taps,
                              **geometry)
     torch.testing.assert_close(q_d.cpu().float(), q_ref.float(), **tol(dtype))
