@@ -57,7 +57,7 @@ __device__ __forceinline__ float load_agent(const float* p) {
 // outputs as one 8-byte load), then the sums in split order.
 template <int N>
 __device__ __forceinline__ unsigned int merge_few(const float* part_o, const float* part_ml, size_t first_part,
-                                                  int splits, int groups, int g, int dim, int d) {
+                                                  int splits, int groups, int g, int dim, int d, float sink2) {
   float m[N], l[N];
   unsigned long long o[N];
 #pragma unroll
@@ -78,6 +78,7 @@ __device__ __forceinline__ unsigned int merge_few(const float* part_o, const flo
     ov0 += f * __uint_as_float((unsigned int)o[sp]);
     ov1 += f * __uint_as_float((unsigned int)(o[sp] >> 32));
   }
+  if (sink2 > -INFINITY) l_tot += __builtin_amdgcn_exp2f(sink2 - m_tot);   // a sink joins the denominator once, here
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   return (unsigned int)float_to_bf16(ov0 * inv) | ((unsigned int)float_to_bf16(ov1 * inv) << 16);
 }
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     float* part_o, float* part_ml, int* __restrict__ counters, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
     int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2,
-    Prepare prep) {
+    Prepare prep, int chunk, const float* __restrict__ sink) {
   constexpr bool PREPARE = MODE != 0, FROM_SUMS = MODE == 2;
   const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
@@ -121,7 +122,10 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   if (cu_q[seq + 1] - q0 != 1) return;
   const int ctx = ctx_len[seq];
   const int cached = PREPARE ? ctx - 1 : ctx;             // keys that the loop below reads from the pages
-  const int k_begin = window > 0 ? max(0, ctx - window) : 0;
+  // the token at position ctx - 1 reads the last `window` keys, and of those the ones of its own
+  // run of `chunk` positions (runs counted from position 0)
+  int k_begin = window > 0 ? max(0, ctx - window) : 0;
+  if (chunk > 0) k_begin = max(k_begin, (ctx - 1) / chunk * chunk);
   const int first = k_begin / KEYS;
   const int last = (cached + KEYS - 1) / KEYS;            // exclusive
   const int per_split = (last - first + splits - 1) / splits;
@@ -489,6 +493,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       }
     }
     if (splits == 1) {
+      // a sink per query head: exp(sink) joins the denominator, with no key and no value
+      if (sink) l += __builtin_amdgcn_exp2f(sink[hk * groups + g] * 1.4426950408889634f - m_tot);
       out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d] = float_to_bf16(l > 0.f ? ov / l : 0.f);
     } else {
       const size_t slot = ((size_t)seq * kv_heads + hk) * splits + split;
@@ -533,9 +539,10 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     for (int e = 2 * tid; e < groups * D; e += 512) {
       const int g = e / D, d = e - g * D;
       unsigned int* dst = (unsigned int*)(out + (size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d);
-      if (splits <= 4) *dst = merge_few<4>(part_o, part_ml, first_part, splits, groups, g, D, d);
-      else if (splits <= 8) *dst = merge_few<8>(part_o, part_ml, first_part, splits, groups, g, D, d);
-      else *dst = merge_few<16>(part_o, part_ml, first_part, splits, groups, g, D, d);
+      const float sink2 = sink ? sink[hk * groups + g] * 1.4426950408889634f : -INFINITY;
+      if (splits <= 4) *dst = merge_few<4>(part_o, part_ml, first_part, splits, groups, g, D, d, sink2);
+      else if (splits <= 8) *dst = merge_few<8>(part_o, part_ml, first_part, splits, groups, g, D, d, sink2);
+      else *dst = merge_few<16>(part_o, part_ml, first_part, splits, groups, g, D, d, sink2);
     }
     return;
   }
@@ -549,6 +556,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       scale_s[g][sp] = f;
       l += f * load_agent(&part_ml[((first_part + sp) * groups + g) * 2 + 1]);
     }
+    if (sink) l += __builtin_amdgcn_exp2f(sink[hk * groups + g] * 1.4426950408889634f - m_tot);
     inv_l[g] = l > 0.f ? 1.f / l : 0.f;
   }
   __syncthreads();
@@ -565,7 +573,7 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
                          const int* cu_q, const int* ctx_len, const int* block_table, int table_stride,
                          int num_seqs, int kv_heads, int groups, int head_dim, int block_size,
                          int num_blocks, int window, float scale, int splits, const Prepare* prep,
-                         hipStream_t stream) {
+                         int chunk, const float* sink, hipStream_t stream) {
   if (num_seqs <= 0) return FE_OK;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
   if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
@@ -576,13 +584,14 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
   if ((((uintptr_t)out) & 3) || (((uintptr_t)part_o) & 7)) return FE_BAD_ARGUMENT;   // pairs of outputs, pairs of partial sums
   if ((((uintptr_t)q) | ((uintptr_t)key_pages) | ((uintptr_t)value_pages)) & 15) return FE_BAD_ARGUMENT;
   if (splits > 1 && (!part_o || !part_ml || !counters)) return FE_BAD_ARGUMENT;
+  if (chunk < 0) return FE_BAD_ARGUMENT;
   dim3 grid(splits, kv_heads, num_seqs);
   const float scale_log2 = scale * 1.4426950408889634f;
   const Prepare none = {nullptr, nullptr, nullptr, 0.f, nullptr, 0, 0};
 #define FE_GO(DD, MODE)                                                                                    \
   paged_decode_kernel<DD, MODE><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none)
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none, chunk, sink)
   if (prep && prep->num_sums > 0) {
     if (head_dim == 64) FE_GO(64, 2);
     else if (head_dim == 128) FE_GO(128, 2);
@@ -615,7 +624,23 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
                                          int splits, hipStream_t stream) {
   return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
                        ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
-                       num_blocks, window, scale, splits, nullptr, stream);
+                       num_blocks, window, scale, splits, nullptr, 0, nullptr, stream);
+}
+
+// The same with the masks and softmax forms beyond the causal one: `chunk` > 0: the token reads
+// keys of its own run of `chunk` positions only (runs counted from position 0); `sink` (float32
+// [kv_heads * groups], or null): exp(sink_h) joins head h's softmax denominator, with no key and
+// no value.
+extern "C" int fe_paged_attention_decode_masked(const void* q, long long q_stride, const void* key_pages,
+                                                const void* value_pages, void* out, long long out_stride,
+                                                float* part_o, float* part_ml, int* counters, const int* cu_q,
+                                                const int* ctx_len, const int* block_table, int table_stride,
+                                                int num_seqs, int kv_heads, int groups, int head_dim,
+                                                int block_size, int num_blocks, int window, int chunk,
+                                                const float* sink, float scale, int splits, hipStream_t stream) {
+  return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
+                       ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
+                       num_blocks, window, scale, splits, nullptr, chunk, sink, stream);
 }
 
 // The same for a batch in which EVERY sequence brings one token, straight from the fused
@@ -644,5 +669,5 @@ extern "C" int fe_paged_attention_decode_prepare(const void* qkv, int qkv_sums, 
   const Prepare prep = {q_weight, k_weight, inv_freq, eps, qkv_sums > 0 ? (const float*)qkv : nullptr, qkv_sums, sum_stride};
   return launch_decode(qkv, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
                        ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
-                       num_blocks, window, scale, splits, &prep, stream);
+                       num_blocks, window, scale, splits, &prep, 0, nullptr, stream);
 }

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
-    float scale_log2, int num_seqs, int heads_per_xcd) {
+    float scale_log2, int num_seqs, int heads_per_xcd, int chunk, const float* __restrict__ sink) {
   const int block_mask = (1 << block_shift) - 1;
   constexpr int BM = 64 * RM;
   constexpr int KC = D / 32;            // MFMA k-steps over the head dim (scores)
@@ -242,7 +242,14 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
   const int last_row = min(q_len, row0 + BM) - 1;
   const int pos_lo = before + row0, pos_hi = before + last_row;
   const int wave_lo = pos_lo + wave * 16 * RM;      // the position of the wave's first row; its last: + 16 RM - 1
-  const int k_first = window > 0 ? max(0, pos_lo - window + 1) : 0;
+  // `chunk` > 0: a row reads keys of its own run of `chunk` positions only (runs counted from
+  // position 0); the block's first row has the lowest such bound, its last row the highest
+  int k_first = window > 0 ? max(0, pos_lo - window + 1) : 0;
+  if (chunk > 0) k_first = max(k_first, pos_lo / chunk * chunk);
+  const int run_hi = chunk > 0 ? pos_hi / chunk * chunk : 0;     // keys below this one are hidden from the last row
+  int row_run[RM];
+#pragma unroll
+  for (int rm = 0; rm < RM; ++rm) row_run[rm] = chunk > 0 ? row_pos[rm] / chunk * chunk : 0;
   const int tile_first = k_first / BN, tile_last = pos_hi / BN;   // inclusive
   const int last_key = ctx - 1;
 
@@ -316,14 +323,14 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
   bool moved[RM];
 #pragma unroll
   for (int rm = 0; rm < RM; ++rm) { item_mx[rm] = 0.f; item_m_use[rm] = 0.f; corr[rm] = 1.f; moved[rm] = false; }
-  auto is_edge = [&](int key_base) { return key_base + BN - 1 > wave_lo || (window > 0 && key_base < pos_hi - window + 1); };
+  auto is_edge = [&](int key_base) { return key_base + BN - 1 > wave_lo || (window > 0 && key_base < pos_hi - window + 1) || key_base < run_hi; };
   auto mask_edges = [&](int key_base, floatx4 (&st)[RM][2][2]) {   // one branch a tile, not one a score: the tiles in the middle of a walk skip all of it
 #pragma unroll
     for (int rm = 0; rm < RM; ++rm)
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int key = key_base + 32 * (j >> 3) + 8 * lq + (j & 7);
-        const bool visible = key <= row_pos[rm] && (window <= 0 || key > row_pos[rm] - window);
+        const bool visible = key <= row_pos[rm] && (window <= 0 || key > row_pos[rm] - window) && key >= row_run[rm];
         if (!visible) st[rm][j >> 3][(j >> 2) & 1][j & 3] = -INFINITY;
       }
   };
@@ -586,6 +593,7 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
         const float f_mine = m_run[rm] > -INFINITY ? __builtin_amdgcn_exp2f(m_run[rm] - m_all) : 0.f;
         const float f_other = m_other > -INFINITY ? __builtin_amdgcn_exp2f(m_other - m_all) : 0.f;
         l_run[rm] = l_run[rm] * f_mine + l_other * f_other;
+        m_run[rm] = m_all;      // what the sums now refer to
 #pragma unroll
         for (int t = 0; t < DT; ++t)
 #pragma unroll
@@ -599,6 +607,9 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
 #pragma unroll
   for (int rm = 0; rm < RM; ++rm) {
     if (row[rm] >= q_len) continue;
+    // a sink per query head: exp(sink) joins the denominator, with no key and no value (the sums
+    // refer to m_run, in base-2 units)
+    if (sink) l_run[rm] += __builtin_amdgcn_exp2f(sink[head] * 1.4426950408889634f - m_run[rm]);
     const float inv = l_run[rm] > 0.f ? 1.f / l_run[rm] : 0.f;
     bf16_t* orow = out + (size_t)(q0 + row[rm]) * out_stride + (size_t)head * D;
 #pragma unroll
@@ -617,6 +628,14 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
 // sets of 16 query rows a wave (blocks of 64 or 128 rows); 0 lets the launch choose either, from total_q:
 // the query tokens of all sequences together (the rows of q; the grid is laid out for num_seqs sequences
 // of max_q_len tokens, of which a step with one long portion fills a fraction).
+extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stride, const void* key_pages,
+                                                 const void* value_pages, void* out, long long out_stride,
+                                                 const int* cu_q, const int* ctx_len, const int* block_table,
+                                                 int table_stride, int num_seqs, int max_q_len, int kv_heads,
+                                                 int groups, int head_dim, int block_size, int num_blocks,
+                                                 int window, int chunk, const float* sink, float scale, int key_groups,
+                                                 int row_sets, int total_q, hipStream_t stream);
+
 extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, const void* key_pages,
                                                  const void* value_pages, void* out, long long out_stride,
                                                  const int* cu_q, const int* ctx_len, const int* block_table,
@@ -624,7 +643,24 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
                                                  int groups, int head_dim, int block_size, int num_blocks,
                                                  int window, float scale, int key_groups, int row_sets, int total_q,
                                                  hipStream_t stream) {
+  return fe_paged_attention_prefill_masked(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len, block_table,
+                                           table_stride, num_seqs, max_q_len, kv_heads, groups, head_dim, block_size,
+                                           num_blocks, window, 0, nullptr, scale, key_groups, row_sets, total_q, stream);
+}
+
+// The same with the masks and softmax forms beyond the causal one: `chunk` > 0: a token reads keys
+// of its own run of `chunk` positions only (runs counted from position 0); `sink` (float32
+// [kv_heads * groups], or null): exp(sink_h) joins head h's softmax denominator, with no key and
+// no value.
+extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stride, const void* key_pages,
+                                                 const void* value_pages, void* out, long long out_stride,
+                                                 const int* cu_q, const int* ctx_len, const int* block_table,
+                                                 int table_stride, int num_seqs, int max_q_len, int kv_heads,
+                                                 int groups, int head_dim, int block_size, int num_blocks,
+                                                 int window, int chunk, const float* sink, float scale, int key_groups,
+                                                 int row_sets, int total_q, hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
+  if (chunk < 0) return FE_BAD_ARGUMENT;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
   if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
   if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
@@ -660,7 +696,7 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
 #define FE_GO(DD, GG, RR)                                                                                            \
   paged_prefill_kernel<DD, GG, RR><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
-      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd)
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink)
 #define FE_GO_D(DD)                                          \
   if (key_groups == 1 && row_sets == 1) FE_GO(DD, 1, 1);      \
   else if (row_sets == 1) FE_GO(DD, 2, 1);                    \

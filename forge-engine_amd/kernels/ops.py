@@ -713,8 +713,14 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                     ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
                     window: int | None = None, num_decode: int | None = None,
-                    max_ctx: int | None = None, splits: int | None = None) -> Tensor:
+                    max_ctx: int | None = None, splits: int | None = None, chunk: int | None = None,
+                    sink: Tensor | None = None) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
+
+    ``chunk`` (a token reads keys of its own run of that many positions only) and ``sink``
+    (float32 [Hq]: exp(sink_h) joins head h's softmax denominator) are served by the two
+    matrix-core kernels alone: a call that brings either for sizes those do not take is refused
+    (``masked_attention`` routes such sizes to the vector-ALU kernel that knows both).
 
     q: [T, >= Hq*D] (row stride may exceed Hq*D: the q part of a fused qkv
     buffer); out [T, Hq*D]; cu_q int32 [B+1]; ctx_len int32 [B] (keys after the
@@ -758,6 +764,16 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                   and q.data_ptr() % 16 == 0 and q_stride % 8 == 0)      # the fast kernels read 16 bytes at a time
     fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
     fast_prefill = bf16_pages and head_dim in (64, 128)
+    masked = chunk is not None or sink is not None
+    if masked:
+        if (any_single and not fast_decode) or (any_longer and not fast_prefill):
+            raise KernelError("chunks and sinks are served by the matrix-core attention kernels only")
+        if sink is not None:
+            _gpu(sink, "sink", torch.float32)
+            if sink.shape != (q_heads,):
+                raise KernelError(f"sink must be [{q_heads}]")
+        if chunk is not None and chunk < 1:
+            raise KernelError("chunk must be positive")
 
     def general(min_q: int, max_q: int) -> None:
         runs = generic_splits(num_seqs, kv_heads, groups, min(max_q, max_q_len), head_dim, max_ctx)
@@ -775,23 +791,28 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
 
     if any_single and fast_decode:
         if splits is None:
-            splits = decode_splits(num_decode, kv_heads, max_ctx if max_ctx is not None else 16 * 4 * 8)
+            reach = max_ctx if max_ctx is not None else 16 * 4 * 8
+            splits = decode_splits(num_decode, kv_heads, reach if chunk is None else min(reach, chunk))
         part_o = part_ml = counters = None
         if splits > 1:
             part_o = torch.empty(num_seqs * kv_heads * splits * groups * head_dim, dtype=torch.float32, device=q.device)
             part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=q.device)
             counters = _split_counters(q.device, num_seqs * kv_heads)
-        _call("attention_decode", "fe_paged_attention_decode", _ptr(q), c_longlong(q_stride),
+        mask = (c_int(chunk or 0), _ptr(sink)) if masked else ()
+        _call("attention_decode", "fe_paged_attention_decode_masked" if masked else "fe_paged_attention_decode",
+              _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(part_o),
               _ptr(part_ml), _ptr(counters), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
               c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(splits), _stream())
+              c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), c_int(splits), _stream())
     if any_longer and fast_prefill:
-        _call("attention_prefill", "fe_paged_attention_prefill", _ptr(q), c_longlong(q_stride),
+        mask = (c_int(chunk or 0), _ptr(sink)) if masked else ()
+        _call("attention_prefill", "fe_paged_attention_prefill_masked" if masked else "fe_paged_attention_prefill",
+              _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(PREFILL_KEY_GROUPS), c_int(PREFILL_ROW_SETS),
+              c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), c_int(PREFILL_KEY_GROUPS), c_int(PREFILL_ROW_SETS),
               c_int(tokens), _stream())
     # whatever the two fast kernels did not take: single tokens go to the vector-ALU decode kernel where
     # it can read four elements at a time, the rest to the general kernel
@@ -1219,13 +1240,17 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
 def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor, ctx_len: Tensor,
                      block_table: Tensor, *, num_seqs: int, max_q_len: int, q_heads: int, kv_heads: int, head_dim: int,
                      value_dim: int, scale: float, window: int | None = None, chunk: int | None = None,
-                     sink: Tensor | None = None, gate: Tensor | None = None) -> Tensor:
+                     sink: Tensor | None = None, gate: Tensor | None = None, num_decode: int | None = None,
+                     max_ctx: int | None = None) -> Tensor:
     """Paged grouped-query attention with the masks and softmax forms beyond the causal one: the
     query at position p reads keys j <= p with j > p - window (``window``) and j >= p - p % chunk
     (``chunk``); ``sink`` (float32 [Hq]) adds exp(sink_h) to head h's softmax denominator, with
     no key and no value; values may be of another width than keys; ``gate`` ([T, Hq * Dv] rows of
     any stride) multiplies the result by sigmoid(gate).  out [T, Hq * Dv].  Scores and softmax
-    float32."""
+    float32.  A bfloat16 cache with keys and values of 64 or 128 elements, groups up to 8 and pages of
+    a power of two >= 16 goes to the matrix-core kernels of ``paged_attention`` (single tokens and
+    portions each to its own), with the gate in a small kernel behind them; everything else, and
+    the float32 mode, to the vector-ALU kernel that does all of it in one launch."""
     _gpu(q, "q", contiguous=False)
     _gpu(out, "out", q.dtype)
     _gpu(key_pages, "key_pages", q.dtype)
@@ -1259,6 +1284,15 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
             raise KernelError("gate must be in q's dtype")
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
+    if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
+            and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
+        paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
+                        q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
+                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink)
+        if gate is not None:
+            _call("stream_ops", "fe_sigmoid_gate", _ptr(out), _ptr(gate), c_longlong(gate_stride), c_int(_code(out.dtype)),
+                  c_int(tokens), c_int(q_heads * value_dim), _stream())
+        return out
     _call("attention_masked", "fe_masked_attention", _ptr(q), c_int(_code(q.dtype)), c_longlong(q_stride), _ptr(key_pages),
           _ptr(value_pages), _ptr(out), _ptr(gate), c_longlong(gate_stride), _ptr(sink), _ptr(cu_q), _ptr(ctx_len),
           _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(q_heads),

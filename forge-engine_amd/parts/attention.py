@@ -244,7 +244,8 @@ class GroupedQueryAttention(Mixer):
             num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim, scale=self.scale,
             window=self.window, chunk=self.chunk, sink=self.sink_weight,
-            gate=qkv[:, self.conv_channels:] if self.output_gate else None)
+            gate=qkv[:, self.conv_channels:] if self.output_gate else None, num_decode=batch.num_decode,
+            max_ctx=batch.max_ctx)
         update = ops.linear_update(attn, self.o_weight)
         return update if self.o_bias_f32 is None else ops.add_bias(update, self.o_bias_f32)
 
@@ -261,7 +262,7 @@ class GroupedQueryAttention(Mixer):
 
     def kernel_libraries(self):
         if self.general:
-            return {"conv_rope", "attention_masked", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+            return {"conv_rope", "attention_masked", "attention_decode", "attention_prefill", "stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
         return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 
 

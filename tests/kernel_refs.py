@@ -413,7 +413,7 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
 
 
 def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, q_heads, kv_heads,
-                     head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None):
+                     head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None, num_decode=None, max_ctx=None):
     block_size = key_pages.shape[2]
     groups = q_heads // kv_heads
     for s in range(num_seqs):

@@ -185,13 +185,15 @@ def ops():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("chunk,block_size", [(24, 16), (7, 4), (64, 8)])
-def test_a_key_just_outside_the_chunk_is_not_seen_and_one_just_inside_is(ops, dtype, chunk, block_size):
+@pytest.mark.parametrize("chunk,block_size", [(24, 16), (7, 4), (64, 8), (80, 32)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 32, 16), (4, 2, 64, 64), (8, 1, 128, 128)])
+def test_a_key_just_outside_the_chunk_is_not_seen_and_one_just_inside_is(ops, dtype, chunk, block_size, heads, kv_heads, dim, vdim):
     """Keys whose scores would dominate sit just before every chunk's first position and at it;
     the attention kernel is compared with the plain chunked attention, for a prompt's portion and
-    for single tokens, and the sink alone is seen by a chunk's first token."""
+    for single tokens, and the sink alone is seen by a chunk's first token.  Heads of 64 and 128 in
+    bfloat16 with pages of 16 or more take the matrix-core kernels, the others the vector-ALU one."""
     g = torch.Generator().manual_seed(chunk)
-    heads, kv_heads, dim, vdim, length = 4, 2, 32, 16, 3 * chunk + 5
+    length = 3 * chunk + 5
     q = torch.randn(length, heads, dim, generator=g)
     k = torch.randn(length, kv_heads, dim, generator=g)
     v = torch.randn(length, kv_heads, vdim, generator=g)
@@ -199,7 +201,7 @@ def test_a_key_just_outside_the_chunk_is_not_seen_and_one_just_inside_is(ops, dt
         k[edge - 1] *= 8.0          # the last key of the chunk before: outside for every token from `edge` on
         k[edge] *= 4.0              # the chunk's first key: inside
     q, k, v = (t.to(dtype) for t in (q, k, v))
-    sink = torch.tensor([0.5, -1.0, 3.0, 0.0])
+    sink = torch.tensor([0.5, -1.0, 3.0, 0.0, 6.0, -4.0, 1.0, 2.0])[:heads]
     positions = torch.arange(length)
     want = plain.chunked_sink_attention(q.double(), k.double(), v.double(), positions, scale=0.4, chunk=chunk,
                                         sink=sink.double()).reshape(length, heads * vdim).float()
