@@ -8,21 +8,22 @@
 // (value-major) and is carried from step to step, so a request may be cut into steps anywhere; a
 // step may hold portions of prompts beside single tokens.
 //
-// Work split: block = (16 value columns, head, sequence), 256 threads.  Thread (rg = tid % 16,
+// Work split: block = (8 value columns, head, sequence), 128 threads.  Thread (rg = tid % 16,
 // jl = tid / 16) owns column jl of the block and the R key channels rg * R .. rg * R + R - 1 of that
 // column's state in registers for the whole walk; the 16 lanes of a column meet by lane permutes.
-// Tokens are staged 16 at a time through LDS (q, k, decay per key channel with its transform
-// applied, v times the input scale), so the exponentials of the decays are computed by all threads
-// at once and the walk itself is multiply-adds.  A block's columns are its own, so nothing is
-// shared between blocks and the state is read once and written once per step.
-// Decays: kind 1  a = exp(-exp(d + bias)),  kind 2  a = sigmoid(d + bias)^(1 / tau) =
-// exp(logsigmoid(d + bias) / tau); times a per-head factor where given.  One more column fed by
-// v = 1 (`ones_column`) follows the recurrence with k alone: a normaliser.
+// Tokens are staged a chunk (16, or 8 for key sizes beyond 128) at a time through LDS: q, k, the
+// decay per key channel with its transform applied, v times the input scale, the per-head decay.
+// The exponentials of the decays are thus computed by all threads at once and the walk itself is
+// multiply-adds.  The next chunk's loads are issued into registers before the walk over this
+// chunk begins, so that memory latency hides behind the walk.  A block's columns are its own, so
+// nothing is shared between blocks and the state is read once and written once per step.
+// Decays: per key channel, kind 1  a = exp(-exp(d + bias)),  kind 2  a = sigmoid(d + bias)^(1 / tau)
+// = exp(logsigmoid(d + bias) / tau); or one factor per head and token (not both).  One more
+// column fed by v = 1 (`ones_column`) follows the recurrence with k alone: a normaliser.
 #include "common.h"
 
-#define LR_THREADS 256
-#define LR_COLS 16
-#define LR_CHUNK 16
+#define LR_THREADS 128
+#define LR_COLS 8
 
 __device__ __forceinline__ float sum_16_lanes(float v) {
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // lane ^ 1
@@ -48,13 +49,19 @@ struct RecurrenceArgs {
   int is_bf16, decay_kind, ones_column, slots, heads, key_dim, value_dim, tokens;
 };
 
-template <int R, bool BONUS>
+// CHANNEL: the decay comes per key channel (p.decay with its transform); else per head and token
+// (p.head_decay, or none at all: 1).
+template <int R, bool BONUS, bool CHANNEL>
 __global__ __launch_bounds__(LR_THREADS) void linear_recurrence_kernel(RecurrenceArgs p) {
   constexpr int DKP = 16 * R;                  // key channels, padded
-  __shared__ float Qs[LR_CHUNK][DKP];
-  __shared__ float Ks[LR_CHUNK][DKP];
-  __shared__ float As[LR_CHUNK][DKP];
-  __shared__ float Vs[LR_CHUNK][LR_COLS];
+  constexpr int CH = R > 8 ? 8 : 16;           // tokens a chunk
+  constexpr int E = CH * DKP / LR_THREADS;     // elements of a chunk's q (and k, and decay) a thread stages
+  __shared__ float Qs[CH][DKP];
+  __shared__ float Ks[CH][DKP];
+  __shared__ float As[CHANNEL ? CH : 1][DKP];
+  __shared__ float Vs[CH][LR_COLS];
+  __shared__ float Hd[CH];
+  __shared__ float Bs[DKP];
 
   const int seq = blockIdx.z, h = blockIdx.y, j0 = blockIdx.x * LR_COLS;
   const int begin = p.cu_q[seq], end = p.cu_q[seq + 1];
@@ -74,54 +81,72 @@ __global__ __launch_bounds__(LR_THREADS) void linear_recurrence_kernel(Recurrenc
     S[m] = (col < columns && i < Dk) ? mine[i] : 0.f;
     U[m] = (BONUS && i < Dk) ? p.bonus[(size_t)h * Dk + i] : 0.f;
   }
+  if (CHANNEL)
+    for (int i = tid; i < DKP; i += LR_THREADS) Bs[i] = i < Dk ? p.decay_bias[(size_t)h * Dk + i] : 0.f;
 
-  for (int t0 = begin; t0 < end; t0 += LR_CHUNK) {
-    __syncthreads();     // the chunk before is consumed
-    for (int e = tid; e < LR_CHUNK * DKP; e += LR_THREADS) {
+  // a chunk's loads, into registers: every load is unconditional (indices past the end are clamped, what
+  // they bring is dropped when the chunk is staged)
+  float qr[E], kr[E], dr[CHANNEL ? E : 1], vr = 0.f, sr = 1.f, hr = 1.f;
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int n = 0; n < E; ++n) {
+      const int e = tid + n * LR_THREADS;
       const int tt = e / DKP, i = e - tt * DKP;
-      const int t = t0 + tt;
-      float qv = 0.f, kv = 0.f, av = 1.f;
-      if (t < end && i < Dk) {
-        const size_t c = (size_t)h * Dk + i;
-        qv = load_either(p.q, (size_t)t * p.q_stride + c, is_bf16) * p.q_scale;
-        kv = load_either(p.k, (size_t)t * p.k_stride + c, is_bf16);
-        if (p.decay_kind == 1) {
-          av = expf(-expf(p.decay[(size_t)t * H * Dk + c] + p.decay_bias[c]));
-        } else if (p.decay_kind == 2) {
-          av = expf(log_sigmoid(p.decay[(size_t)t * H * Dk + c] + p.decay_bias[c]) / p.tau);
-        }
-        if (p.head_decay) av *= p.head_decay[(size_t)t * H + h];
-      }
-      Qs[tt][i] = qv;
-      Ks[tt][i] = kv;
-      As[tt][i] = av;
+      const size_t t = (size_t)min(t0 + tt, end - 1);
+      const size_t c = (size_t)h * Dk + min(i, Dk - 1);
+      qr[n] = load_either(p.q, t * p.q_stride + c, is_bf16);
+      kr[n] = load_either(p.k, t * p.k_stride + c, is_bf16);
+      if (CHANNEL) dr[n] = p.decay[t * H * Dk + c];
     }
-    for (int e = tid; e < LR_CHUNK * LR_COLS; e += LR_THREADS) {
-      const int tt = e / LR_COLS, j = e - tt * LR_COLS;
-      const int t = t0 + tt, c = j0 + j;
-      float vv = 0.f;
-      if (t < end) {
-        if (c < Dv) vv = load_either(p.v, (size_t)t * p.v_stride + (size_t)h * Dv + c, is_bf16);
-        else if (c < columns) vv = 1.f;
-        if (p.in_scale) vv *= p.in_scale[(size_t)t * H + h];
-      }
-      Vs[tt][j] = vv;
+    if (tid < CH * LR_COLS) {
+      const int tt = tid / LR_COLS, c = j0 + tid % LR_COLS;
+      const size_t t = (size_t)min(t0 + tt, end - 1);
+      vr = load_either(p.v, t * p.v_stride + (size_t)h * Dv + min(c, Dv - 1), is_bf16);
+      if (c >= Dv) vr = c < columns ? 1.f : 0.f;
+      sr = p.in_scale ? p.in_scale[t * H + h] : 1.f;
     }
-    __syncthreads();
+    if (tid < CH) hr = p.head_decay ? p.head_decay[(size_t)min(t0 + tid, end - 1) * H + h] : 1.f;
+  };
+  auto stage = [&](int t0) {
+#pragma unroll
+    for (int n = 0; n < E; ++n) {
+      const int e = tid + n * LR_THREADS;
+      const int tt = e / DKP, i = e - tt * DKP;
+      const bool live = t0 + tt < end && i < Dk;
+      Qs[tt][i] = live ? qr[n] * p.q_scale : 0.f;
+      Ks[tt][i] = live ? kr[n] : 0.f;
+      if (CHANNEL) {
+        const float z = dr[n] + Bs[i];
+        const float a = p.decay_kind == 1 ? expf(-expf(z)) : expf(log_sigmoid(z) / p.tau);
+        As[tt][i] = live ? a : 1.f;
+      }
+    }
+    if (tid < CH * LR_COLS) Vs[tid / LR_COLS][tid % LR_COLS] = t0 + tid / LR_COLS < end ? vr * sr : 0.f;
+    if (tid < CH) Hd[tid] = hr;
+  };
 
-    const int count = min(LR_CHUNK, end - t0);
+  fetch(begin);
+  for (int t0 = begin; t0 < end; t0 += CH) {
+    __syncthreads();     // the chunk before is consumed (and the bias row is in place)
+    stage(t0);
+    __syncthreads();
+    if (t0 + CH < end) fetch(t0 + CH);      // in flight while this chunk is walked
+
+    const int count = min(CH, end - t0);
     for (int tt = 0; tt < count; ++tt) {
       const float vj = Vs[tt][jl];
+      const float hd = CHANNEL ? 1.f : Hd[tt];
       float acc = 0.f;
 #pragma unroll
       for (int m = 0; m < R; ++m) {
         const int i = rg * R + m;
         const float kv = Ks[tt][i] * vj;
+        const float a = CHANNEL ? As[tt][i] : hd;
         if (BONUS) {
           acc = fmaf(fmaf(U[m], kv, S[m]), Qs[tt][i], acc);
-          S[m] = fmaf(S[m], As[tt][i], kv);
+          S[m] = fmaf(S[m], a, kv);
         } else {
-          S[m] = fmaf(S[m], As[tt][i], kv);
+          S[m] = fmaf(S[m], a, kv);
           acc = fmaf(S[m], Qs[tt][i], acc);
         }
       }
@@ -141,8 +166,10 @@ __global__ __launch_bounds__(LR_THREADS) void linear_recurrence_kernel(Recurrenc
 
 template <int R>
 static void launch_recurrence(const RecurrenceArgs& p, dim3 grid, hipStream_t stream) {
-  if (p.bonus) linear_recurrence_kernel<R, true><<<grid, LR_THREADS, 0, stream>>>(p);
-  else linear_recurrence_kernel<R, false><<<grid, LR_THREADS, 0, stream>>>(p);
+  if (p.bonus && p.decay_kind) linear_recurrence_kernel<R, true, true><<<grid, LR_THREADS, 0, stream>>>(p);
+  else if (p.bonus) linear_recurrence_kernel<R, true, false><<<grid, LR_THREADS, 0, stream>>>(p);
+  else if (p.decay_kind) linear_recurrence_kernel<R, false, true><<<grid, LR_THREADS, 0, stream>>>(p);
+  else linear_recurrence_kernel<R, false, false><<<grid, LR_THREADS, 0, stream>>>(p);
 }
 
 extern "C" int fe_linear_recurrence(const void* q, const void* k, const void* v, int dtype, long long q_stride,
@@ -154,7 +181,7 @@ extern "C" int fe_linear_recurrence(const void* q, const void* k, const void* v,
   if (tokens <= 0 || num_seqs <= 0) return FE_OK;
   if (heads <= 0 || key_dim < 1 || key_dim > 256 || value_dim < 1 || slots < 1 || max_q_len < 1 ||
       (dtype != FE_F32 && dtype != FE_BF16) || decay_kind < 0 || decay_kind > 2 || (decay_kind && (!decay || !decay_bias)) ||
-      !(tau > 0.f) || heads > 65535 || num_seqs > 65535)
+      !(tau > 0.f) || heads > 65535 || num_seqs > 65535 || (decay_kind && head_decay))
     return FE_BAD_ARGUMENT;
   if (q_stride < (long long)heads * key_dim || k_stride < (long long)heads * key_dim || v_stride < (long long)heads * value_dim)
     return FE_BAD_ARGUMENT;

@@ -1316,8 +1316,8 @@ def linear_recurrence(q: Tensor, k: Tensor, v: Tensor, out: Tensor, state: Tenso
     key_dim] (value-major) between steps.
 
     a_t per key channel from ``decay`` (float32 [T, heads * key_dim], before its bias):
-    ``exp_neg_exp`` a = exp(-exp(d + bias)), ``sigmoid_root`` a = sigmoid(d + bias)^(1 / tau); times
-    ``head_decay`` (float32 [T, heads]) where given; b_t = ``in_scale`` [T, heads] or 1.
+    ``exp_neg_exp`` a = exp(-exp(d + bias)), ``sigmoid_root`` a = sigmoid(d + bias)^(1 / tau); or per
+    head from ``head_decay`` (float32 [T, heads]; not both); b_t = ``in_scale`` [T, heads] or 1.
     ``bonus`` (float32 [heads * key_dim]): the query reads the state before the token's update plus
     diag(bonus) k_t v_t^T instead.  ``ones_column``: one more value column fed by v = 1 (a
     normaliser).  q, k [T, heads * key_dim] and v [T, heads * value_dim] rows of any stride, in the
@@ -1350,6 +1350,8 @@ def linear_recurrence(q: Tensor, k: Tensor, v: Tensor, out: Tensor, state: Tenso
         raise KernelError(f"bonus must hold {heads * key_dim} entries")
     if decay is not None and decay_bias is None:
         raise KernelError("a decay comes with its bias")
+    if decay is not None and head_decay is not None:
+        raise KernelError("the decay comes per key channel or per head, not both")
     if max_q_len < 1 or not tau > 0.0:
         raise KernelError("max_q_len and tau must be positive")
     _call("linear_recurrence", "fe_linear_recurrence", _ptr(q), _ptr(k), _ptr(v), c_int(_code(q.dtype)),
