@@ -1320,7 +1320,8 @@ def linear_recurrence(q: Tensor, k: Tensor, v: Tensor, out: Tensor, state: Tenso
     head from ``head_decay`` (float32 [T, heads]; not both); b_t = ``in_scale`` [T, heads] or 1.
     ``bonus`` (float32 [heads * key_dim]): the query reads the state before the token's update plus
     diag(bonus) k_t v_t^T instead.  ``ones_column``: one more value column fed by v = 1 (a
-    normaliser).  q, k [T, heads * key_dim] and v [T, heads * value_dim] rows of any stride, in the
+    normaliser).  ``decay`` is overwritten with the decays a_t (its transform runs in place, in a
+    kernel of its own over the whole step, before the walk).  q, k [T, heads * key_dim] and v [T, heads * value_dim] rows of any stride, in the
     compute dtype; out float32 [T, heads, value_dim (+1)]."""
     columns = value_dim + (1 if ones_column else 0)
     tokens = q.shape[0]
