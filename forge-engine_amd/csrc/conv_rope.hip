@@ -8,13 +8,15 @@
 // its last taps - 1 projected rows; a second kernel moves the state on after the first has read it.
 // The projection's bias (float32, one entry per q, k and v channel, or none) is added here, to the
 // rows as they are loaded, so that the product before this kernel has none; the state holds rows
-// with their bias.  One block per token; everything between the loads and the stores is float32.
+// with their bias.  One wave per token and head; everything between the loads and the stores is float32.
 #include "common.h"
 
 #define CR_THREADS 256
+#define CR_HEAD_MAX 256
 
+// One wave per (token, head): q heads, then k heads, then v heads.
 template <typename T>
-__global__ __launch_bounds__(CR_THREADS) void conv_rope_norm_write_kernel(
+__global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
     const T* __restrict__ qkv, size_t qkv_stride, const float* __restrict__ bias, const float* __restrict__ conv_w,
     const float* __restrict__ conv_state, const float* __restrict__ inv_freq,
     const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ cu_q,
@@ -22,78 +24,77 @@ __global__ __launch_bounds__(CR_THREADS) void conv_rope_norm_write_kernel(
     T* __restrict__ key_pages, T* __restrict__ value_pages, T* __restrict__ q_out, int q_heads, int kv_heads,
     int head_dim, int value_dim, int rotary_dim, float eps, int unit_norm, int taps, int block_size,
     int num_blocks, int slots) {
-  extern __shared__ float y[];   // [channels]
-  const int t = blockIdx.x;
-  const int tid = threadIdx.x;
+  __shared__ float y[CR_HEAD_MAX];
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int seq = token_seq[t];
   const int begin = cu_q[seq];
   const int pos = positions[t];
   const int q_size = q_heads * head_dim, k_size = kv_heads * head_dim, v_size = kv_heads * value_dim;
   const int channels = q_size + k_size + v_size;
+  const bool is_q = head < q_heads, is_v = head >= q_heads + kv_heads;
+  const int n = is_v ? value_dim : head_dim;
+  const int first = is_q ? head * head_dim
+                         : (is_v ? q_size + k_size + (head - q_heads - kv_heads) * value_dim : q_size + (head - q_heads) * head_dim);
 
-  // 1. convolution (or a plain copy) into LDS
-  if (taps > 0) {
-    const int slot = min(max(state_slots[seq], 0), slots - 1);
-    const float* kept = conv_state + (size_t)slot * (taps - 1) * channels;
-    for (int c = tid; c < channels; c += CR_THREADS) {
-      float acc = 0.f;
-      const float b = bias ? bias[c] : 0.f;
+  // 1. the head's channels: bias, convolution over the rows of this step and of the state
+  const int slot = taps > 0 ? min(max(state_slots[seq], 0), slots - 1) : 0;
+  const float* kept = taps > 0 ? conv_state + (size_t)slot * (taps - 1) * channels : nullptr;
+  for (int d = lane; d < n; d += 64) {
+    const int c = first + d;
+    const float b = bias ? bias[c] : 0.f;
+    float acc;
+    if (taps > 0) {
+      acc = 0.f;
       for (int j = 0; j < taps; ++j) {
         const int row = t - (taps - 1) + j;          // a row of this step, or of the state if before `begin`
         const float u = row >= begin ? load_as_float(qkv + (size_t)row * qkv_stride + c) + b
                                      : kept[(size_t)(taps - 1 - (begin - row)) * channels + c];
         acc = fmaf(conv_w[(size_t)c * taps + j], u, acc);
       }
-      y[c] = acc;
+    } else {
+      acc = load_as_float(qkv + (size_t)t * qkv_stride + c) + b;
     }
-  } else {
-    for (int c = tid; c < channels; c += CR_THREADS)
-      y[c] = load_as_float(qkv + (size_t)t * qkv_stride + c) + (bias ? bias[c] : 0.f);
+    y[d] = acc;
   }
   __syncthreads();
 
-  // 2. rotation of q and k heads, a pair per thread
-  const int half = rotary_dim / 2;
-  const int rot_heads = q_heads + kv_heads;
-  for (int e = tid; e < rot_heads * half; e += CR_THREADS) {
-    const int head = e / half, i = e - head * half;
-    float sn, cs;
-    sincosf((float)pos * inv_freq[i], &sn, &cs);
-    float* hv = y + head * head_dim;
-    const float a = hv[i], b = hv[i + half];
-    hv[i] = a * cs - b * sn;
-    hv[i + half] = b * cs + a * sn;
-  }
-  __syncthreads();
-
-  // 3. unit norm per head and the stores: a wave per head
-  const int lane = tid & 63, wave = tid >> 6;
   const int page = block_table[(size_t)seq * table_stride + pos / block_size];
   const int place = pos % block_size;
   const bool paged = page >= 0 && page < num_blocks;
-  for (int head = wave; head < rot_heads; head += CR_THREADS / 64) {
-    const float* hv = y + head * head_dim;
-    float inv = 1.f;
-    if (unit_norm) {
-      float ss = 0.f;
-      for (int c = lane; c < head_dim; c += 64) ss += hv[c] * hv[c];
-      ss = wave_sum(ss);
-      inv = rsqrtf(ss / (float)head_dim + eps);
+  if (is_v) {
+    if (paged) {
+      const int hv = head - q_heads - kv_heads;
+      for (int d = lane; d < n; d += 64)
+        store_from_float(value_pages + (((size_t)page * kv_heads + hv) * value_dim + d) * block_size + place, y[d]);
     }
-    if (head < q_heads) {
-      T* dst = q_out + (size_t)t * q_size + head * head_dim;
-      for (int c = lane; c < head_dim; c += 64) store_from_float(dst + c, hv[c] * inv);
-    } else if (paged) {
-      T* dst = key_pages + (((size_t)page * kv_heads + (head - q_heads)) * block_size + place) * head_dim;
-      for (int c = lane; c < head_dim; c += 64) store_from_float(dst + c, hv[c] * inv);
-    }
+    return;
   }
-  if (paged) {
-    const float* vv = y + q_size + k_size;
-    for (int e = tid; e < v_size; e += CR_THREADS) {
-      const int head = e / value_dim, d = e - head * value_dim;
-      store_from_float(value_pages + (((size_t)page * kv_heads + head) * value_dim + d) * block_size + place, vv[e]);
-    }
+
+  // 2. rotation, a pair per lane
+  const int half = rotary_dim / 2;
+  for (int i = lane; i < half; i += 64) {
+    float sn, cs;
+    sincosf((float)pos * inv_freq[i], &sn, &cs);
+    const float a = y[i], b = y[i + half];
+    y[i] = a * cs - b * sn;
+    y[i + half] = b * cs + a * sn;
+  }
+  __syncthreads();
+
+  // 3. unit norm and the store
+  float inv = 1.f;
+  if (unit_norm) {
+    float ss = 0.f;
+    for (int d = lane; d < n; d += 64) ss += y[d] * y[d];
+    ss = wave_sum(ss);
+    inv = rsqrtf(ss / (float)head_dim + eps);
+  }
+  if (is_q) {
+    T* dst = q_out + (size_t)t * q_size + head * head_dim;
+    for (int d = lane; d < n; d += 64) store_from_float(dst + d, y[d] * inv);
+  } else if (paged) {
+    T* dst = key_pages + (((size_t)page * kv_heads + (head - q_heads)) * block_size + place) * head_dim;
+    for (int d = lane; d < n; d += 64) store_from_float(dst + d, y[d] * inv);
   }
 }
 
@@ -137,10 +138,11 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
   if (taps < 0 || taps == 1 || taps > 8 || (taps && (!conv_w || !conv_state || slots < 1))) return FE_BAD_ARGUMENT;
   if (unit_norm && !(eps > 0.f)) return FE_BAD_ARGUMENT;
   const long long channels = (long long)(q_heads + kv_heads) * head_dim + (long long)kv_heads * value_dim;
-  if (channels > 16000 || qkv_stride < channels) return FE_BAD_ARGUMENT;      // a token's channels live in LDS
-  const size_t lds = (size_t)channels * sizeof(float);
+  if (head_dim > CR_HEAD_MAX || value_dim > CR_HEAD_MAX || qkv_stride < channels || q_heads + 2 * kv_heads > 65535)
+    return FE_BAD_ARGUMENT;      // a head lives in LDS
+  const dim3 grid(tokens, q_heads + 2 * kv_heads);
 #define LAUNCH(T)                                                                                              \
-  conv_rope_norm_write_kernel<T><<<tokens, CR_THREADS, lds, stream>>>(                                         \
+  conv_rope_norm_write_kernel<T><<<grid, 64, 0, stream>>>(                                         \
       (const T*)qkv, (size_t)qkv_stride, bias, conv_w, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, \
       block_table, table_stride, (T*)key_pages, (T*)value_pages, (T*)q_out, q_heads, kv_heads, head_dim,       \
       value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots)

@@ -7,6 +7,9 @@
 #include "common.h"
 
 #define ROW_THREADS 256
+#define ROW_THREADS_FEW 1024   // threads a row when a step has few rows (measured faster up to some hundred rows)
+#define FEW_ROWS 512
+static inline int row_threads(int rows, int width) { return rows <= FEW_ROWS && width >= 1024 ? ROW_THREADS_FEW : ROW_THREADS; }
 
 template <typename T>
 __device__ __forceinline__ T* as(void* p) { return (T*)p; }
@@ -15,7 +18,7 @@ __device__ __forceinline__ T* as(void* p) { return (T*)p; }
 // out[s][t][c] = x[t][c] + (prev[t][c] - x[t][c]) * w[s][c]; prev = x[t - 1] inside the token's
 // sequence, the sequence's state row for its first token of the step.
 template <typename TX, typename TO>
-__global__ __launch_bounds__(ROW_THREADS) void token_shift_kernel(
+__global__ __launch_bounds__(ROW_THREADS_FEW) void token_shift_kernel(
     const TX* __restrict__ x, const float* __restrict__ w, const float* __restrict__ state,
     const int* __restrict__ cu_q, const int* __restrict__ token_seq, const int* __restrict__ state_slots,
     TO* __restrict__ out, int tokens, int width, int count, int slots) {
@@ -26,7 +29,7 @@ __global__ __launch_bounds__(ROW_THREADS) void token_shift_kernel(
   const TX* row = x + (size_t)t * width;
   const TX* before = first ? row : row - width;   // never an address before the buffer
   const float* kept = state + (size_t)min(max(slot, 0), slots - 1) * width;
-  for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float v = load_as_float(row + c);
     const float p = first ? kept[c] : load_as_float(before + c);
     const float d = p - v;
@@ -55,7 +58,7 @@ extern "C" int fe_token_shift(const void* x, int x_dtype, const float* weights, 
   if (tokens <= 0) return FE_OK;
   if (width <= 0 || count < 1 || count > 8 || slots < 1) return FE_BAD_ARGUMENT;
 #define LAUNCH(TX, TO)                                                                                       \
-  token_shift_kernel<TX, TO><<<tokens, ROW_THREADS, 0, stream>>>((const TX*)x, weights, state, cu_q, token_seq, \
+  token_shift_kernel<TX, TO><<<tokens, row_threads(tokens, width), 0, stream>>>((const TX*)x, weights, state, cu_q, token_seq, \
                                                                   state_slots, (TO*)out, tokens, width, count, slots)
   if (x_dtype == FE_F32 && out_dtype == FE_F32) LAUNCH(float, float);
   else if (x_dtype == FE_F32 && out_dtype == FE_BF16) LAUNCH(float, bf16_t);
@@ -86,24 +89,49 @@ __device__ __forceinline__ float parts_sum(const float* p, int parts, size_t par
 }
 
 // h[r] += u * rsqrt(mean(u^2) + eps) * w, u = the sum of the update's parts; out (if any) = new h.
+// A row of up to 8 elements a thread stays in registers between the two passes (the parts are read
+// once); wider rows are read again.
 template <typename TO, bool HAS_OUT>
-__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_update_kernel(
+__global__ __launch_bounds__(ROW_THREADS_FEW) void rmsnorm_update_kernel(
     float* __restrict__ h, const float* __restrict__ update, int parts, size_t part_stride,
     const float* __restrict__ w, float eps, TO* __restrict__ out, int width) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * width;
+  const int threads = blockDim.x;
+  const bool held = width <= 8 * threads;
+  float u[8];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
-    const float u = parts_sum(update + base + c, parts, part_stride);
-    ss += u * u;
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = threadIdx.x + j * threads;
+      u[j] = c < width ? parts_sum(update + base + c, parts, part_stride) : 0.f;
+      ss += u[j] * u[j];
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += threads) {
+      const float v = parts_sum(update + base + c, parts, part_stride);
+      ss += v * v;
+    }
   }
   ss = block_sum<true>(ss, scratch);
   const float inv = rsqrtf(ss / (float)width + eps);
-  for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
-    const float u = parts_sum(update + base + c, parts, part_stride);
-    const float v = h[base + c] + u * inv * w[c];
-    h[base + c] = v;
-    if (HAS_OUT) store_from_float(out + base + c, v);
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = threadIdx.x + j * threads;
+      if (c < width) {
+        const float v = h[base + c] + u[j] * inv * w[c];
+        h[base + c] = v;
+        if (HAS_OUT) store_from_float(out + base + c, v);
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += threads) {
+      const float v = h[base + c] + parts_sum(update + base + c, parts, part_stride) * inv * w[c];
+      h[base + c] = v;
+      if (HAS_OUT) store_from_float(out + base + c, v);
+    }
   }
 }
 
@@ -112,11 +140,11 @@ extern "C" int fe_rmsnorm_update(float* h, const float* update, int parts, long 
   if (rows <= 0) return FE_OK;
   if (width <= 0 || parts < 1 || parts > 64 || !(eps > 0.f)) return FE_BAD_ARGUMENT;
   if (out == nullptr || out_dtype < 0)
-    rmsnorm_update_kernel<float, false><<<rows, ROW_THREADS, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, nullptr, width);
+    rmsnorm_update_kernel<float, false><<<rows, row_threads(rows, width), 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, nullptr, width);
   else if (out_dtype == FE_F32)
-    rmsnorm_update_kernel<float, true><<<rows, ROW_THREADS, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, (float*)out, width);
+    rmsnorm_update_kernel<float, true><<<rows, row_threads(rows, width), 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, (float*)out, width);
   else if (out_dtype == FE_BF16)
-    rmsnorm_update_kernel<bf16_t, true><<<rows, ROW_THREADS, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, (bf16_t*)out, width);
+    rmsnorm_update_kernel<bf16_t, true><<<rows, row_threads(rows, width), 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, (bf16_t*)out, width);
   else return FE_BAD_ARGUMENT;
   return fe_check_launch();
 }
@@ -127,7 +155,7 @@ struct MeanInputs {
   int parts[4];
 };
 
-__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_mean_kernel(MeanInputs in, int count, size_t part_stride,
+__global__ __launch_bounds__(ROW_THREADS_FEW) void rmsnorm_mean_kernel(MeanInputs in, int count, size_t part_stride,
                                                                    const float* __restrict__ w, float eps,
                                                                    float* __restrict__ out, int width) {
   __shared__ float scratch[4][16];
@@ -135,7 +163,7 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_mean_kernel(MeanInputs in
   float inv[4];
   for (int b = 0; b < count; ++b) {
     float ss = 0.f;
-    for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
       const float u = parts_sum(in.u[b] + base + c, in.parts[b], part_stride);
       ss += u * u;
     }
@@ -143,7 +171,7 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_mean_kernel(MeanInputs in
     inv[b] = rsqrtf(ss / (float)width + eps);
   }
   const float share = 1.f / (float)count;
-  for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float total = 0.f;
     for (int b = 0; b < count; ++b)
       total += parts_sum(in.u[b] + base + c, in.parts[b], part_stride) * inv[b] * w[(size_t)b * width + c];
@@ -159,19 +187,19 @@ extern "C" int fe_rmsnorm_mean(const float* u0, const float* u1, const float* u2
   MeanInputs in = {{u0, u1, u2, u3}, {p0, p1, p2, p3}};
   for (int b = 0; b < count; ++b)
     if (in.u[b] == nullptr || in.parts[b] < 1 || in.parts[b] > 64) return FE_BAD_ARGUMENT;
-  rmsnorm_mean_kernel<<<rows, ROW_THREADS, 0, stream>>>(in, count, (size_t)part_stride, w, eps, out, width);
+  rmsnorm_mean_kernel<<<rows, row_threads(rows, width), 0, stream>>>(in, count, (size_t)part_stride, w, eps, out, width);
   return fe_check_launch();
 }
 
 // ---------------------------------------------------------------- PolyNorm
 // out = a z/rms(z) + b z^2/rms(z^2) + c z^3/rms(z^3) + e over a row
 template <typename T>
-__global__ __launch_bounds__(ROW_THREADS) void polynorm_kernel(const T* __restrict__ z, const float* __restrict__ coeff,
+__global__ __launch_bounds__(ROW_THREADS_FEW) void polynorm_kernel(const T* __restrict__ z, const float* __restrict__ coeff,
                                                                float eps, T* __restrict__ out, int width) {
   __shared__ float scratch[3][16];
   const size_t base = (size_t)blockIdx.x * width;
   float s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float v = load_as_float(z + base + c);
     const float v2 = v * v;
     s1 += v2;
@@ -184,7 +212,7 @@ __global__ __launch_bounds__(ROW_THREADS) void polynorm_kernel(const T* __restri
   const float n = (float)width;
   const float a = coeff[0] * rsqrtf(s1 / n + eps), b = coeff[1] * rsqrtf(s2 / n + eps),
               c3 = coeff[2] * rsqrtf(s3 / n + eps), e = coeff[3];
-  for (int c = threadIdx.x; c < width; c += ROW_THREADS) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float v = load_as_float(z + base + c);
     const float v2 = v * v;
     store_from_float(out + base + c, a * v + b * v2 + c3 * (v2 * v) + e);
@@ -196,9 +224,9 @@ extern "C" int fe_polynorm(const void* z, int dtype, const float* coeff, float e
   if (rows <= 0) return FE_OK;
   if (width <= 0 || !(eps > 0.f)) return FE_BAD_ARGUMENT;
   if (dtype == FE_F32)
-    polynorm_kernel<float><<<rows, ROW_THREADS, 0, stream>>>((const float*)z, coeff, eps, (float*)out, width);
+    polynorm_kernel<float><<<rows, row_threads(rows, width), 0, stream>>>((const float*)z, coeff, eps, (float*)out, width);
   else if (dtype == FE_BF16)
-    polynorm_kernel<bf16_t><<<rows, ROW_THREADS, 0, stream>>>((const bf16_t*)z, coeff, eps, (bf16_t*)out, width);
+    polynorm_kernel<bf16_t><<<rows, row_threads(rows, width), 0, stream>>>((const bf16_t*)z, coeff, eps, (bf16_t*)out, width);
   else return FE_BAD_ARGUMENT;
   return fe_check_launch();
 }
