@@ -37,8 +37,8 @@ __global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
                          : (is_v ? q_size + k_size + (head - q_heads - kv_heads) * value_dim : q_size + (head - q_heads) * head_dim);
 
   // 1. the head's channels: bias, convolution over the rows of this step and of the state
-  const int slot = taps > 0 ? min(max(state_slots[seq], 0), slots - 1) : 0;
-  const float* kept = taps > 0 ? conv_state + (size_t)slot * (taps - 1) * channels : nullptr;
+  const int slot = taps > 1 ? min(max(state_slots[seq], 0), slots - 1) : 0;
+  const float* kept = taps > 1 ? conv_state + (size_t)slot * (taps - 1) * channels : nullptr;    // one tap reads no earlier row
   for (int d = lane; d < n; d += 64) {
     const int c = first + d;
     const float b = bias ? bias[c] : 0.f;
@@ -135,7 +135,7 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
   if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || value_dim <= 0 || block_size <= 0 || num_blocks <= 0)
     return FE_BAD_ARGUMENT;
   if (rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 || (rotary_dim && !inv_freq)) return FE_BAD_ARGUMENT;
-  if (taps < 0 || taps == 1 || taps > 8 || (taps && (!conv_w || !conv_state || slots < 1))) return FE_BAD_ARGUMENT;
+  if (taps < 0 || taps > 8 || (taps && !conv_w) || (taps > 1 && (!conv_state || slots < 1))) return FE_BAD_ARGUMENT;
   if (unit_norm && !(eps > 0.f)) return FE_BAD_ARGUMENT;
   const long long channels = (long long)(q_heads + kv_heads) * head_dim + (long long)kv_heads * value_dim;
   if (head_dim > CR_HEAD_MAX || value_dim > CR_HEAD_MAX || qkv_stride < channels || q_heads + 2 * kv_heads > 65535)

@@ -1177,7 +1177,7 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
     projection's bias (float32 [channels] or None: the product before has none), a short causal
     convolution over time on every q, k and v channel (``taps`` > 0: y_t = sum_j c[:, j] *
     u_(t - taps + 1 + j), rows before the step from ``conv_state`` [slots, taps - 1, channels],
-    which afterwards holds every sequence's last taps - 1 projected rows); rotation of the first
+    which afterwards holds every sequence's last taps - 1 projected rows; one tap needs no state); rotation of the first
     ``rotary_dim`` dims of q and k heads (dim i pairs with i + rotary_dim / 2); then q and k heads
     divided by their root mean square (``unit_norm_eps`` not None); q into ``q_out`` [T, Hq * D],
     k and v into their pages (values transposed).  float32 inside, one rounding at the stores.
@@ -1196,9 +1196,10 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
             raise KernelError(f"bias must be [{channels}]")
     if taps:
         _gpu(conv_weight, "conv_weight", torch.float32)
+        if conv_weight.shape != (channels, taps) or not 1 <= taps <= 8:
+            raise KernelError(f"conv_weight must be [{channels}, taps in 1..8]")
+    if taps > 1:
         _gpu(conv_state, "conv_state", torch.float32)
-        if conv_weight.shape != (channels, taps) or not 2 <= taps <= 8:
-            raise KernelError(f"conv_weight must be [{channels}, taps in 2..8]")
         if conv_state.dim() != 3 or conv_state.shape[1:] != (taps - 1, channels):
             raise KernelError(f"conv_state must be [slots, {taps - 1}, {channels}]")
     if rotary_dim:
@@ -1223,15 +1224,15 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
     if block_table.dim() != 2 or block_table.stride(1) != 1 or block_table.shape[0] < num_seqs:
         raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
     stride = qkv.stride(0) if tokens > 1 else max(qkv.stride(0), qkv.shape[1])
-    slots = conv_state.shape[0] if taps else 0
+    slots = conv_state.shape[0] if taps > 1 else 0
     _call("conv_rope", "fe_conv_rope_norm_write", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias),
-          _ptr(conv_weight if taps else None), _ptr(conv_state if taps else None), _ptr(inv_freq if rotary_dim else None),
+          _ptr(conv_weight if taps else None), _ptr(conv_state if taps > 1 else None), _ptr(inv_freq if rotary_dim else None),
           _ptr(positions), _ptr(token_seq), _ptr(cu_q), _ptr(state_slots), _ptr(block_table), c_int(block_table.stride(0)),
           _ptr(key_pages), _ptr(value_pages), _ptr(q_out), c_int(tokens), c_int(q_heads), c_int(kv_heads), c_int(head_dim),
           c_int(value_dim), c_int(rotary_dim), c_float(unit_norm_eps if unit_norm_eps is not None else 0.0),
           c_int(1 if unit_norm_eps is not None else 0), c_int(taps), c_int(block_size), c_int(num_blocks), c_int(slots),
           _stream())
-    if taps:
+    if taps > 1:
         _call("conv_rope", "fe_conv_state_update", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias), _ptr(conv_state),
               _ptr(cu_q), _ptr(state_slots), c_int(num_seqs), c_int(channels), c_int(taps), c_int(slots), c_int(tokens),
               _stream())

@@ -60,8 +60,8 @@ class GroupedQueryAttention(Mixer):
         self.chunk = chunk
         self.sink = sink
         self.output_gate = output_gate
-        if self.conv_taps == 1 or self.conv_taps < 0:
-            raise ValueError("a short convolution has at least two taps (0: none)")
+        if self.conv_taps < 0:
+            raise ValueError("a short convolution has at least one tap (0: none)")
         if chunk is not None and (chunk < 1 or window is not None):
             raise ValueError("chunk must be positive and cannot be combined with a window")
         # the general path: anything the fused kernels of the plain arrangement do not know
@@ -179,7 +179,7 @@ class GroupedQueryAttention(Mixer):
     def cache_needs(self) -> CacheNeeds:
         paged = PagedKV(self.num_kv_heads, self.head_dim, self.window,
                         None if self.value_dim == self.head_dim else self.value_dim, chunk=self.chunk)
-        if not self.conv_taps:
+        if self.conv_taps < 2:        # one tap looks at the token's own row only: nothing to keep
             return CacheNeeds(paged=paged)
         # the last taps - 1 projected rows (q, k and v channels), exact in float32
         return CacheNeeds(paged=paged, state={self.CONV_STATE: FixedState((self.conv_taps - 1, self.conv_channels), torch.float32)})
@@ -233,7 +233,7 @@ class GroupedQueryAttention(Mixer):
         qkv = ops.linear(x, self.qkv_weight)        # [T, q | k | v (| gate)]; the bias is added by the kernel below
         q = torch.empty((x.shape[0], self.q_size), dtype=x.dtype, device=x.device)
         ops.conv_rope_norm_write(
-            qkv, self.conv_bias, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps else None, inv_freq,
+            qkv, self.conv_bias, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps > 1 else None, inv_freq,
             batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
             cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,

@@ -383,6 +383,9 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
             a, b = int(cu_q[s]), int(cu_q[s + 1])
             if b == a:
                 continue
+            if taps == 1:
+                y[a:b] = u[a:b] * conv_weight[:, 0]
+                continue
             slot = int(state_slots[s])
             history = torch.cat([conv_state[slot], u[a:b]])            # [taps - 1 + n, channels]
             y[a:b] = sum(history[j:j + b - a] * conv_weight[:, j] for j in range(taps))

@@ -42,6 +42,8 @@ ALONE = {
     "gla": config(64, 32, [layer("gla", GLA_Q, None)]),
     "mlstm": config(64, 32, [layer("mlstm", MLSTM_P, None)]),
     "feed_forward": config(64, 32, [layer("gla", GLA_P, 50)]),
+    # one tap (a scale per channel, no state), one head, two rotated dims, a chunk of one position (a token sees itself and the sink)
+    "one_tap": config(64, 32, [layer("parallel", {"left": attention(1, 1, 16, 16, 1, 1, 2), "right": {"heads": 2, "dim": 8, "rank": 1}}, 40)]),
 }
 BLOCK_SIZE = {"A": 4, "B": 8}
 

@@ -150,6 +150,7 @@ def attention_case(g, dtype, lengths, before, *, q_heads, kv_heads, head_dim, va
     dict(q_heads=4, kv_heads=2, head_dim=64, value_dim=64, block_size=16, taps=4, rotary_dim=64),
     dict(q_heads=3, kv_heads=3, head_dim=24, value_dim=40, block_size=4, taps=2, rotary_dim=12),
     dict(q_heads=6, kv_heads=2, head_dim=128, value_dim=32, block_size=8, taps=0, rotary_dim=0),
+    dict(q_heads=2, kv_heads=1, head_dim=256, value_dim=72, block_size=16, taps=1, rotary_dim=2),
 ])
 def test_conv_rope_norm_write(ops, dtype, sizes):
     g = torch.Generator().manual_seed(8)
@@ -165,7 +166,7 @@ def test_conv_rope_norm_write(ops, dtype, sizes):
     qkv = wide[:, :channels]
     bias = rand(g, channels) if sizes["value_dim"] != 32 else None
     conv_w = rand(g, channels, taps) if taps else None
-    state = rand(g, 6, taps - 1, channels) if taps else None
+    state = rand(g, 6, taps - 1, channels) if taps > 1 else None
     inv_freq = (1.0 / 10000.0 ** (torch.arange(0, rotary_dim, 2).float() / rotary_dim)) if rotary_dim else None
     state_ref = None if state is None else state.clone()
     keys_ref, values_ref = keys.clone(), values.clone()
@@ -181,7 +182,7 @@ def test_conv_rope_norm_write(ops, dtype, sizes):
     torch.testing.assert_close(q_d.cpu().float(), q_ref.float(), **tol(dtype))
     torch.testing.assert_close(keys_d.cpu().float(), keys_ref.float(), **tol(dtype))
     torch.testing.assert_close(values_d.cpu().float(), values_ref.float(), **tol(dtype))
-    if taps:
+    if taps > 1:
         torch.testing.assert_close(state_d.cpu(), state_ref, atol=0, rtol=0)
 
 
