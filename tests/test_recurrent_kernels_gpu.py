@@ -147,7 +147,7 @@ def attention_case(g, dtype, lengths, before, *, q_heads, kv_heads, head_dim, va
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [
-    dict(q_heads=4, kv_heads=2, head_dim=64, value_dim=64, block_size=16, taps=4, rotary_dim=64),
+    dict(q_heads=6, kv_heads=3, head_dim=64, value_dim=64, block_size=16, taps=3, rotary_dim=32),
     dict(q_heads=3, kv_heads=3, head_dim=24, value_dim=40, block_size=4, taps=2, rotary_dim=12),
     dict(q_heads=6, kv_heads=2, head_dim=128, value_dim=32, block_size=8, taps=0, rotary_dim=0),
     dict(q_heads=2, kv_heads=1, head_dim=256, value_dim=72, block_size=16, taps=1, rotary_dim=2),
@@ -188,7 +188,8 @@ def test_conv_rope_norm_write(ops, dtype, sizes):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [
-    dict(q_heads=4, kv_heads=2, head_dim=64, value_dim=64, block_size=16, chunk=24, window=None, sink=True, gate=True),
+    dict(q_heads=8, kv_heads=2, head_dim=64, value_dim=64, block_size=16, chunk=24, window=None, sink=True, gate=True),
+    dict(q_heads=6, kv_heads=2, head_dim=128, value_dim=128, block_size=32, chunk=33, window=None, sink=True, gate=True),
     dict(q_heads=3, kv_heads=3, head_dim=24, value_dim=40, block_size=4, chunk=7, window=None, sink=True, gate=False),
     dict(q_heads=6, kv_heads=1, head_dim=128, value_dim=16, block_size=8, chunk=None, window=11, sink=False, gate=True),
     dict(q_heads=2, kv_heads=2, head_dim=200, value_dim=130, block_size=16, chunk=1000, window=None, sink=True, gate=False),
@@ -215,7 +216,7 @@ def test_masked_attention(ops, dtype, sizes):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("form", ["rwkv", "gla", "mlstm", "plain"])
-@pytest.mark.parametrize("heads,key_dim,value_dim", [(4, 32, 32), (2, 48, 64), (3, 20, 50), (1, 128, 16), (2, 200, 24)])
+@pytest.mark.parametrize("heads,key_dim,value_dim", [(5, 32, 32), (2, 48, 80), (3, 20, 50), (1, 128, 16), (2, 200, 24), (3, 64, 40), (2, 136, 9)])
 def test_linear_recurrence(ops, dtype, form, heads, key_dim, value_dim):
     g = torch.Generator().manual_seed(10)
     lengths = [5, 0, 1, 37, 2]
