@@ -185,7 +185,7 @@ def ops():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("chunk,block_size", [(24, 16), (7, 4), (64, 8), (80, 32)])
+@pytest.mark.parametrize("chunk,block_size", [(24, 16), (7, 4), (64, 8), (80, 32), (5, 16)])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 32, 16), (6, 3, 64, 64), (8, 1, 128, 128)])
 def test_a_key_just_outside_the_chunk_is_not_seen_and_one_just_inside_is(ops, dtype, chunk, block_size, heads, kv_heads, dim, vdim):
     """Keys whose scores would dominate sit just before every chunk's first position and at it;
