@@ -11,9 +11,6 @@
 #define FEW_ROWS 512
 static inline int row_threads(int rows, int width) { return rows <= FEW_ROWS && width >= 1024 ? ROW_THREADS_FEW : ROW_THREADS; }
 
-template <typename T>
-__device__ __forceinline__ T* as(void* p) { return (T*)p; }
-
 // ---------------------------------------------------------------- token shift
 // out[s][t][c] = x[t][c] + (prev[t][c] - x[t][c]) * w[s][c]; prev = x[t - 1] inside the token's
 // sequence, the sequence's state row for its first token of the step.

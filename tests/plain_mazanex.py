@@ -31,10 +31,6 @@ def token_shift(h, weight):
     return h + (previous_rows(h) - h) * weight
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def short_convolution(u, taps_weight):
     """u [T, C], taps_weight [C, K]: y_t = sum_j w[:, j] * u_(t - K + 1 + j), zeros before the start."""
     T, C = u.shape
