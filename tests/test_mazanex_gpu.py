@@ -29,9 +29,17 @@ WIDE = mu.config(300, 128, [
     mu.layer("parallel", {"left": mu.attention(4, 1, 64, 32, 4, 48, 32, scale=0.11), "right": {"heads": 2, "dim": 64, "rank": 8}}, 160),
     mu.layer("mlstm", {"heads": 2, "dim": 32, "vdim": 128, "gate_cap": 10.0}, None),
 ])
-CONFIGS = {"A": mu.MIXED_A, "B": mu.MIXED_B, "W": WIDE}
-LENGTHS = {"A": (5, 1, 14, 27, 90), "B": (2, 9, 21, 33, 64), "W": (3, 50, 130, 97, 200)}
-BLOCKS = {"A": 4, "B": 8, "W": 16}
+# keys and values of 128 in groups of two (in bfloat16 the matrix-core attention kernels serve it, chunks and sink
+# included), key sizes of 128 and 136 in the recurrences (a wave per column of the state), a one-tap neighbour
+MATRIX = mu.config(210, 160, [
+    mu.layer("parallel", {"left": mu.attention(4, 2, 128, 128, 2, 40, 64, scale=0.09), "right": {"heads": 2, "dim": 128, "rank": 6}}, 200),
+    mu.layer("mlstm", {"heads": 2, "dim": 136, "vdim": 24, "gate_cap": 9.0}, 120),
+    mu.layer("gla", {"heads": 1, "dim": 128, "vdim": 72, "tau": 20.0, "rank": 4}, None),
+    mu.layer("parallel", {"left": mu.attention(2, 2, 64, 64, 1, 33, 16, scale=0.12), "right": {"heads": 5, "dim": 16, "rank": 2}}, 96),
+])
+CONFIGS = {"A": mu.MIXED_A, "B": mu.MIXED_B, "W": WIDE, "M": MATRIX}
+LENGTHS = {"A": (5, 1, 14, 27, 90), "B": (2, 9, 21, 33, 64), "W": (3, 50, 130, 97, 200), "M": (4, 45, 150, 83, 1)}
+BLOCKS = {"A": 4, "B": 8, "W": 16, "M": 16}
 
 
 @pytest.fixture(scope="module")
