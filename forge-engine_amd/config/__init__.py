@@ -4,6 +4,7 @@ from .engine import EngineConfig, SchedulerConfig
 from .model import ConfigError, ModelConfig, load_model_config
 from .mazanex import MazanexConfig
 from .qwen3 import Qwen3Config
+from .rekezen import RekezenConfig
 
-__all__ = ["ConfigError", "EngineConfig", "MazanexConfig", "ModelConfig", "Qwen3Config", "SchedulerConfig",
+__all__ = ["ConfigError", "EngineConfig", "MazanexConfig", "ModelConfig", "Qwen3Config", "RekezenConfig", "SchedulerConfig",
            "load_model_config"]

@@ -5,7 +5,8 @@
 //   * a sink per query head: exp(sink_h) joins the softmax's denominator, with no key and no value
 //     (the running maximum starts at sink_h and the running sum at 1);
 //   * values of another width than keys;
-//   * an output gate: the result times sigmoid(gate).
+//   * an output gate: the result times sigmoid(gate), a gate per element or one per query head;
+//   * a soft cap: scores, after the scale, become cap * tanh(score / cap).
 // One launch serves portions of prompts and single tokens alike; the step's own keys and values are
 // already in the pages (keys [page][kv head][slot][D], values transposed [page][kv head][Dv][slot]).
 // Block = (tile of 16 rows, kv head, sequence), a row being a (query token, head of the group) pair,
@@ -22,7 +23,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     T* __restrict__ out, const T* __restrict__ gate, size_t gate_stride, const float* __restrict__ sink,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int D, int Dv, int block_size, int num_blocks, int window,
-    int chunk, float scale) {
+    int chunk, float scale, float softcap, int head_gate) {
   constexpr int KPT = TK / 16;
   extern __shared__ float smem[];
   const int ks = D + 1, vs = Dv + 1;
@@ -117,7 +118,9 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     for (int i = 0; i < KPT; ++i) {
       const int kp = kt + c + 16 * i;
       const bool visible = row_ok && kp <= my_pos && kp >= my_first;
-      s[i] = visible ? s[i] * scale : -INFINITY;
+      float score = s[i] * scale;
+      if (softcap > 0.f) score = softcap * tanhf(score / softcap);
+      s[i] = visible ? score : -INFINITY;
       tile_max = fmaxf(tile_max, s[i]);
     }
 #pragma unroll
@@ -158,13 +161,14 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     const float inv = l > 0.f ? 1.f / l : 0.f;
     const size_t at = (size_t)head * Dv;
     T* orow = out + (size_t)(q0 + my_tok) * ((size_t)kv_heads * groups * Dv) + at;
-    const T* grow = gate ? gate + (size_t)(q0 + my_tok) * gate_stride + at : nullptr;
+    const T* grow = gate ? gate + (size_t)(q0 + my_tok) * gate_stride + (head_gate ? (size_t)head : at) : nullptr;
+    const float whole = (grow && head_gate) ? 1.f / (1.f + expf(-load_as_float(grow))) : 1.f;
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
       const int d = c + 16 * i;
       if (d < Dv) {
-        float v = acc[i] * inv;
-        if (grow) v *= 1.f / (1.f + expf(-load_as_float(grow + d)));
+        float v = acc[i] * inv * whole;
+        if (grow && !head_gate) v *= 1.f / (1.f + expf(-load_as_float(grow + d)));
         store_from_float(orow + d, v);
       }
     }
@@ -176,7 +180,7 @@ static int launch_masked(const void* q, long long q_stride, const void* key_page
                          const void* gate, long long gate_stride, const float* sink, const int* cu_q,
                          const int* ctx_len, const int* block_table, int table_stride, int num_seqs, int max_q_len,
                          int q_heads, int kv_heads, int D, int Dv, int block_size, int num_blocks, int window,
-                         int chunk, float scale, hipStream_t stream) {
+                         int chunk, float scale, float softcap, int head_gate, hipStream_t stream) {
   const int groups = q_heads / kv_heads;
   const long long rows = (long long)max_q_len * groups;
   const dim3 grid((unsigned)((rows + ROWS - 1) / ROWS), kv_heads, num_seqs);
@@ -186,7 +190,7 @@ static int launch_masked(const void* q, long long q_stride, const void* key_page
   masked_attention_kernel<T, TK, DPT><<<grid, 256, lds, stream>>>(                                               \
       (const T*)q, (size_t)q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, (const T*)gate,        \
       (size_t)gate_stride, sink, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, D, Dv, block_size, \
-      num_blocks, window, chunk, scale)
+      num_blocks, window, chunk, scale, softcap, head_gate)
   if (tk == 32) {
     if (Dv <= 64) LAUNCH(32, 4);
     else if (Dv <= 128) LAUNCH(32, 8);
@@ -205,21 +209,22 @@ extern "C" int fe_masked_attention(const void* q, int dtype, long long q_stride,
                                    const float* sink, const int* cu_q, const int* ctx_len, const int* block_table,
                                    int table_stride, int num_seqs, int max_q_len, int q_heads, int kv_heads,
                                    int head_dim, int value_dim, int block_size, int num_blocks, int window, int chunk,
-                                   float scale, int tokens, hipStream_t stream) {
+                                   float scale, float softcap, int head_gate, int tokens, hipStream_t stream) {
   if (tokens <= 0 || num_seqs <= 0) return FE_OK;
   if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || head_dim < 1 || head_dim > 256 || value_dim < 1 ||
       value_dim > 256 || block_size <= 0 || num_blocks <= 0 || max_q_len < 1 || window < 0 || chunk < 0 ||
       num_seqs > 65535 || kv_heads > 65535)
     return FE_BAD_ARGUMENT;
-  if (q_stride < (long long)q_heads * head_dim || (gate && gate_stride < (long long)q_heads * value_dim))
+  if (q_stride < (long long)q_heads * head_dim || softcap < 0.f ||
+      (gate && gate_stride < (long long)q_heads * (head_gate ? 1 : value_dim)))
     return FE_BAD_ARGUMENT;
   if (dtype == FE_F32)
     return launch_masked<float>(q, q_stride, key_pages, value_pages, out, gate, gate_stride, sink, cu_q, ctx_len,
                                 block_table, table_stride, num_seqs, max_q_len, q_heads, kv_heads, head_dim, value_dim,
-                                block_size, num_blocks, window, chunk, scale, stream);
+                                block_size, num_blocks, window, chunk, scale, softcap, head_gate, stream);
   if (dtype == FE_BF16)
     return launch_masked<bf16_t>(q, q_stride, key_pages, value_pages, out, gate, gate_stride, sink, cu_q, ctx_len,
                                  block_table, table_stride, num_seqs, max_q_len, q_heads, kv_heads, head_dim, value_dim,
-                                 block_size, num_blocks, window, chunk, scale, stream);
+                                 block_size, num_blocks, window, chunk, scale, softcap, head_gate, stream);
   return FE_BAD_ARGUMENT;
 }

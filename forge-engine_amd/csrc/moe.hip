@@ -1,0 +1,279 @@
+// A mixture of experts on the device: routing, the sort of (token, choice) pairs by expert, and
+// two grouped matrix products over the sorted rows.  Nothing is decided on the host.
+//
+//   fe_moe_route:    z = W_r x + b (float32), the `top` largest per token, softmax over those alone
+//   fe_moe_plan:     counts per expert, their prefix sums, and the pairs ordered by expert
+//   fe_moe_gate_up:  for every pair, act = min(g, L) * sigmoid(alpha min(g, L)) * (clamp(u, -L, L) + 1) with
+//                    g = W_gate[e] x, u = W_up[e] x of the pair's token and expert
+//   fe_moe_down:     out[choice][token] = weight * W_down[e] act   (float32; one part per choice, so
+//                    that the reader adds a token's experts up in a fixed order)
+//   fe_gated_act:    the same activation over a dense [T, 2F] product (a shared expert)
+//
+// The grouped products tile the sorted rows 32 at a time within an expert (a tile never spans two
+// experts) and 64 output columns a block, K through LDS in steps of 32, float32 FMA accumulation.
+// A launch has as many row-tile slots as the pairs could need at worst (pairs / 32 + experts);
+// a block whose slot lies beyond the tiles there are returns at once.
+#include "common.h"
+
+#define ROUTE_WAVES 4
+
+template <typename T>
+__global__ __launch_bounds__(64 * ROUTE_WAVES) void moe_route_kernel(
+    const T* __restrict__ x, const T* __restrict__ router, const float* __restrict__ bias, int* __restrict__ chosen,
+    float* __restrict__ weights, int tokens, int H, int E, int top) {
+  extern __shared__ float logits[];     // [ROUTE_WAVES][E]
+  const int wave = threadIdx.x / FE_WAVE, lane = threadIdx.x % FE_WAVE;
+  const int t = blockIdx.x * ROUTE_WAVES + wave;
+  if (t >= tokens) return;
+  float* z = logits + wave * E;
+  const T* row = x + (size_t)t * H;
+  for (int e = 0; e < E; ++e) {
+    const T* w = router + (size_t)e * H;
+    float partial = 0.f;
+    for (int k = lane; k < H; k += FE_WAVE) partial = fmaf(load_as_float(row + k), load_as_float(w + k), partial);
+    const float total = wave_sum(partial);
+    if (lane == 0) z[e] = total + (bias ? bias[e] : 0.f);
+  }
+  if (lane != 0) return;
+  // the largest first; among equals the lowest index
+  float best[16];
+  float peak = 0.f, denom = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int arg = 0;
+    float value = -INFINITY;
+    for (int e = 0; e < E; ++e)
+      if (z[e] > value) {
+        value = z[e];
+        arg = e;
+      }
+    z[arg] = -INFINITY;
+    chosen[(size_t)t * top + k] = arg;
+    if (k == 0) peak = value;
+    best[k] = expf(value - peak);
+    denom += best[k];
+  }
+  for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] = best[k] / denom;
+}
+
+extern "C" int fe_moe_route(const void* x, const void* router, int dtype, const float* bias, int* chosen, float* weights,
+                            int tokens, int hidden, int experts, int top, hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (hidden <= 0 || experts <= 0 || experts > 1024 || top < 1 || top > 16 || top > experts) return FE_BAD_ARGUMENT;
+  const int blocks = (tokens + ROUTE_WAVES - 1) / ROUTE_WAVES;
+  const size_t lds = (size_t)ROUTE_WAVES * experts * sizeof(float);
+  if (dtype == FE_F32)
+    moe_route_kernel<float><<<blocks, 64 * ROUTE_WAVES, lds, stream>>>((const float*)x, (const float*)router, bias, chosen,
+                                                                       weights, tokens, hidden, experts, top);
+  else if (dtype == FE_BF16)
+    moe_route_kernel<bf16_t><<<blocks, 64 * ROUTE_WAVES, lds, stream>>>((const bf16_t*)x, (const bf16_t*)router, bias, chosen,
+                                                                        weights, tokens, hidden, experts, top);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+// One block: offsets[e] = pairs of experts below e, order[offsets[e] ..] = the pairs of expert e.
+// Within an expert the pairs come in no fixed order; a pair's results do not depend on its row.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int pairs, int E,
+                                                        int* __restrict__ offsets, int* __restrict__ order) {
+  extern __shared__ int counts[];   // [E] counts, then [E] cursors
+  int* cursor = counts + E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = chosen[i];
+    if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sum = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = cursor[e] = sum;
+      sum += counts[e];
+    }
+    offsets[E] = sum;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = chosen[i];
+    if (e >= 0 && e < E) order[atomicAdd(&cursor[e], 1)] = i;
+  }
+}
+
+extern "C" int fe_moe_plan(const int* chosen, int pairs, int experts, int* offsets, int* order, hipStream_t stream) {
+  if (pairs <= 0) return FE_OK;
+  if (experts <= 0 || experts > 1024) return FE_BAD_ARGUMENT;
+  moe_plan_kernel<<<1, 1024, 2 * (size_t)experts * sizeof(int), stream>>>(chosen, pairs, experts, offsets, order);
+  return fe_check_launch();
+}
+
+#define BM 32
+#define BN 64
+#define BK 32
+
+__device__ __forceinline__ float gated(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+}
+
+// The expert and the first sorted row of this block's row tile; false if the slot is beyond the tiles.
+__device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E, int slot, int& expert, int& row0,
+                                          int& row_end) {
+  int tiles = 0;
+  for (int e = 0; e < E; ++e) {
+    const int begin = offsets[e], end = offsets[e + 1];
+    const int mine = (end - begin + BM - 1) / BM;
+    if (slot < tiles + mine) {
+      expert = e;
+      row0 = begin + (slot - tiles) * BM;
+      row_end = end;
+      return true;
+    }
+    tiles += mine;
+  }
+  return false;
+}
+
+// MODE 0: rows are tokens' x gathered through the sorted pairs, the weight is [E][2N][K] (gate rows, then
+// up rows), the ending is the gated activation into act [pairs, N].  MODE 1: rows are act's sorted rows,
+// the weight is [E][N][K], and the result times the pair's routing weight goes to out[choice][token][N].
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void moe_grouped_kernel(
+    const T* __restrict__ a, const T* __restrict__ w, const int* __restrict__ offsets, const int* __restrict__ order,
+    const float* __restrict__ pair_weight, T* __restrict__ act, float* __restrict__ out, int E, int N, int K, int top,
+    int tokens, float limit, float alpha) {
+  __shared__ float As[BM][BK + 1];
+  __shared__ float Ws[BN][BK + 1];
+  __shared__ float Us[MODE == 0 ? BN : 1][BK + 1];
+  __shared__ int pair_of[BM];
+  int expert, row0, row_end;
+  if (!find_tile(offsets, E, blockIdx.x, expert, row0, row_end)) return;
+  const int tid = threadIdx.x;
+  const int n0 = blockIdx.y * BN;
+  if (tid < BM) pair_of[tid] = row0 + tid < row_end ? order[row0 + tid] : -1;
+  __syncthreads();
+  const int ty = tid / 16, tx = tid % 16;
+  float acc_g[2][4], acc_u[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc_g[i][j] = acc_u[i][j] = 0.f;
+  const size_t w_rows = MODE == 0 ? 2 * (size_t)N : (size_t)N;
+  const T* w_expert = w + (size_t)expert * w_rows * K;
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    for (int e = tid; e < BM * BK; e += 256) {
+      const int r = e / BK, k = e % BK;
+      float v = 0.f;
+      const int pair = pair_of[r];
+      if (pair >= 0 && k0 + k < K) {
+        const size_t src = MODE == 0 ? (size_t)(pair / top) : (size_t)(row0 + r);
+        v = load_as_float(a + src * K + k0 + k);
+      }
+      As[r][k] = v;
+    }
+    for (int e = tid; e < BN * BK; e += 256) {
+      const int n = e / BK, k = e % BK;
+      const bool ok = n0 + n < N && k0 + k < K;
+      Ws[n][k] = ok ? load_as_float(w_expert + (size_t)(n0 + n) * K + k0 + k) : 0.f;
+      if (MODE == 0) Us[n][k] = ok ? load_as_float(w_expert + ((size_t)N + n0 + n) * K + k0 + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < BK; ++k) {
+      const float a0 = As[ty * 2][k], a1 = As[ty * 2 + 1][k];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float wv = Ws[tx + 16 * j][k];
+        acc_g[0][j] = fmaf(a0, wv, acc_g[0][j]);
+        acc_g[1][j] = fmaf(a1, wv, acc_g[1][j]);
+        if (MODE == 0) {
+          const float uv = Us[tx + 16 * j][k];
+          acc_u[0][j] = fmaf(a0, uv, acc_u[0][j]);
+          acc_u[1][j] = fmaf(a1, uv, acc_u[1][j]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = ty * 2 + i;
+    const int pair = pair_of[r];
+    if (pair < 0) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n >= N) continue;
+      if (MODE == 0) {
+        store_from_float(act + (size_t)(row0 + r) * N + n, gated(acc_g[i][j], acc_u[i][j], limit, alpha));
+      } else {
+        const int token = pair / top, choice = pair - token * top;
+        out[((size_t)choice * tokens + token) * N + n] = acc_g[i][j] * pair_weight[pair];
+      }
+    }
+  }
+}
+
+extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, const int* offsets, const int* order, void* act,
+                              int tokens, int top, int experts, int hidden, int inner, float limit, float alpha,
+                              hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (top < 1 || experts < 1 || experts > 1024 || hidden <= 0 || inner <= 0 || !(limit > 0.f)) return FE_BAD_ARGUMENT;
+  const long long pairs = (long long)tokens * top;
+  const dim3 grid((unsigned)(pairs / BM + experts), (unsigned)((inner + BN - 1) / BN));
+  if (dtype == FE_F32)
+    moe_grouped_kernel<float, 0><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, offsets, order, nullptr,
+                                                           (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha);
+  else if (dtype == FE_BF16)
+    moe_grouped_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr,
+                                                            (bf16_t*)act, nullptr, experts, inner, hidden, top, tokens, limit,
+                                                            alpha);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+extern "C" int fe_moe_down(const void* act, const void* down, int dtype, const int* offsets, const int* order,
+                           const float* pair_weight, float* out, int tokens, int top, int experts, int hidden, int inner,
+                           hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (top < 1 || experts < 1 || experts > 1024 || hidden <= 0 || inner <= 0) return FE_BAD_ARGUMENT;
+  const long long pairs = (long long)tokens * top;
+  const dim3 grid((unsigned)(pairs / BM + experts), (unsigned)((hidden + BN - 1) / BN));
+  if (dtype == FE_F32)
+    moe_grouped_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, offsets, order, pair_weight,
+                                                           nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f);
+  else if (dtype == FE_BF16)
+    moe_grouped_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight,
+                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+// ---------------------------------------------------------------- the activation over a dense product
+template <typename T>
+__global__ void gated_act_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long long count, int inner, float limit,
+                                 float alpha) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const long long t = i / inner;
+  const int n = (int)(i - t * inner);
+  const T* row = gate_up + t * 2 * inner;
+  store_from_float(out + i, gated(load_as_float(row + n), load_as_float(row + inner + n), limit, alpha));
+}
+
+extern "C" int fe_gated_act(const void* gate_up, void* out, int dtype, int tokens, int inner, float limit, float alpha,
+                            hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (inner <= 0 || !(limit > 0.f)) return FE_BAD_ARGUMENT;
+  const long long count = (long long)tokens * inner;
+  const int blocks = (int)((count + 255) / 256);
+  if (dtype == FE_F32) gated_act_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, count, inner, limit, alpha);
+  else if (dtype == FE_BF16) gated_act_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, count, inner, limit, alpha);
+  else return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}

@@ -209,6 +209,9 @@ class ModelRunner:
         self.states: list[dict[str, Tensor]] = [
             {name: torch.zeros((num_state_slots + 1, *state.shape), dtype=state.dtype or torch.float32, device=self.device)
              for name, state in need.states().items()} for need in needs]
+        self.embedding_states: dict[str, Tensor] = {
+            name: torch.zeros((num_state_slots + 1, *state.shape), dtype=state.dtype or torch.float32, device=self.device)
+            for name, state in model.embedding_needs().states().items()}
         self.pad_state_slot = num_state_slots
         self.steps_run = 0
         self.workspace = ops.Workspace()    # scratch that this runner's launches (and its captured graphs) share
@@ -218,7 +221,7 @@ class ModelRunner:
         """Lease a state slot and empty tables for the request.  The slot's fixed-size state starts
         at zero: the runner clears it here, so a mixer never has to know a request's first step."""
         record = self.cache.begin(request_id)
-        for states in self.states:
+        for states in [*self.states, self.embedding_states]:
             for state in states.values():
                 state[record.state_slot].zero_()
 
@@ -284,6 +287,14 @@ class ModelRunner:
             else:
                 views.append(None)
         return views
+
+    def embedding_view(self, scratch_state: bool = False) -> CacheView | None:
+        """The states of an embedding that keeps some between steps (as a copy for a run whose
+        effects must not stay)."""
+        if not self.embedding_states:
+            return None
+        states = self.embedding_states
+        return CacheView(states={name: state.clone() for name, state in states.items()} if scratch_state else states)
 
     def _graphable(self, entries: list[StepEntry]) -> bool:
         return (self.use_graphs and len(entries) <= GRAPH_MAX_REQUESTS
@@ -361,7 +372,7 @@ class ModelRunner:
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                slot.logits = self.model.forward(batch, views)
+                slot.logits = self.model.forward(batch, views, self.embedding_view())
             slot.graph, slot.views, slot.batch = graph, views, batch
         if device_tokens is not None:
             slot.feed(device_tokens)
@@ -383,7 +394,7 @@ class ModelRunner:
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(side):
-            self.model.forward(batch, views)
+            self.model.forward(batch, views, self.embedding_view(scratch_state=True))
         torch.cuda.current_stream(self.device).wait_stream(side)
 
     def _portion_key(self, entries: list[StepEntry]):
@@ -442,7 +453,7 @@ class ModelRunner:
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                slot.logits = self.model.forward(batch, views)
+                slot.logits = self.model.forward(batch, views, self.embedding_view())
             slot.graph, slot.views, slot.batch = graph, views, batch
         slot.graph.replay()
         self.portion_graph_replays += 1
@@ -485,7 +496,7 @@ class ModelRunner:
             if logits is not None:
                 return logits
         batch = self.prepare(entries)
-        logits = self.model.forward(batch, self.cache_views(batch))
+        logits = self.model.forward(batch, self.cache_views(batch), self.embedding_view())
         for i, entry in enumerate(entries):
             self.cache.commit(entry.request_id, batch.ctx_before_host[i] + batch.q_lens[i])
         self.steps_run += 1

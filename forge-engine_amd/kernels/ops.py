@@ -1242,12 +1242,13 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
                      block_table: Tensor, *, num_seqs: int, max_q_len: int, q_heads: int, kv_heads: int, head_dim: int,
                      value_dim: int, scale: float, window: int | None = None, chunk: int | None = None,
                      sink: Tensor | None = None, gate: Tensor | None = None, num_decode: int | None = None,
-                     max_ctx: int | None = None) -> Tensor:
+                     max_ctx: int | None = None, softcap: float | None = None, head_gate: bool = False) -> Tensor:
     """Paged grouped-query attention with the masks and softmax forms beyond the causal one: the
     query at position p reads keys j <= p with j > p - window (``window``) and j >= p - p % chunk
     (``chunk``); ``sink`` (float32 [Hq]) adds exp(sink_h) to head h's softmax denominator, with
     no key and no value; values may be of another width than keys; ``gate`` ([T, Hq * Dv] rows of
-    any stride) multiplies the result by sigmoid(gate).  out [T, Hq * Dv].  Scores and softmax
+    any stride; with ``head_gate`` [T, Hq], one number a head) multiplies the result by sigmoid(gate);
+    ``softcap``: scores, after the scale, become cap * tanh(score / cap).  out [T, Hq * Dv].  Scores and softmax
     float32.  A bfloat16 cache with keys and values of 64 or 128 elements, groups up to 8 and pages of
     a power of two >= 16 goes to the matrix-core kernels of ``paged_attention`` (single tokens and
     portions each to its own), with the gate in a small kernel behind them; everything else, and
@@ -1280,12 +1281,15 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
             raise KernelError(f"sink must be [{q_heads}]")
     gate_stride = 0
     if gate is not None:
-        gate_stride = _strided_rows(gate, "gate", q_heads * value_dim)
+        gate_stride = _strided_rows(gate, "gate", q_heads if head_gate else q_heads * value_dim)
         if gate.dtype != q.dtype:
             raise KernelError("gate must be in q's dtype")
+    if softcap is not None and not softcap > 0.0:
+        raise KernelError("softcap must be positive")
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
-    if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
+    if (softcap is None and not head_gate
+            and q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
             and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
         paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
                         q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
@@ -1298,7 +1302,8 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
           _ptr(value_pages), _ptr(out), _ptr(gate), c_longlong(gate_stride), _ptr(sink), _ptr(cu_q), _ptr(ctx_len),
           _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(q_heads),
           c_int(kv_heads), c_int(head_dim), c_int(value_dim), c_int(block_size), c_int(num_blocks),
-          c_int(window or 0), c_int(chunk or 0), c_float(scale), c_int(tokens), _stream())
+          c_int(window or 0), c_int(chunk or 0), c_float(scale), c_float(softcap or 0.0), c_int(1 if head_gate else 0),
+          c_int(tokens), _stream())
     return out
 
 
@@ -1384,4 +1389,217 @@ def mlstm_gate_scan(gates: Tensor, bias: Tensor, cap: float, maximum: Tensor, cu
     _call("linear_recurrence", "fe_mlstm_gate_scan", _ptr(gates), _ptr(bias), c_float(cap), _ptr(maximum),
           c_int(maximum.shape[0]), _ptr(cu_q), _ptr(state_slots), _ptr(out), c_int(tokens), c_int(num_seqs), c_int(heads),
           _stream())
+    return out
+
+
+# ------------------------------------------------- several residual streams, token pairs, a factor on the logits
+
+def hyper_norm(streams: Tensor, update: Tensor | None, mix: Tensor | None, share: Tensor | None, read: Tensor | None,
+               weight: Tensor | None, bias: Tensor | None, eps: float, out: Tensor | None, rows: Tensor | None = None,
+               store: bool = True, rms: bool = False) -> Tensor | None:
+    """The norm over S residual streams [S, T, W] (float32; S = 1: one plain stream), fused with the
+    pending update (float32 [T, W] or [parts, T, W], added up in order):
+    ``x_t <- sum_s mix[s, t] x_s + share[t] * update`` (mix None: the identity, share None: ones; written
+    back unless ``store`` is False), ``u = sum_t read[t] x_t`` (None: the plain sum), and ``out`` =
+    the layer norm of u with weight and bias (``rms``: the RMS norm, no mean, bias optional), of the
+    rows listed in ``rows`` if given.  ``out`` None: the update is applied and nothing else."""
+    _gpu(streams, "streams", torch.float32)
+    if streams.dim() != 3 or not 1 <= streams.shape[0] <= 8:
+        raise KernelError(f"streams must be [1..8, T, W], got {tuple(streams.shape)}")
+    count, total_rows, width = streams.shape
+    if width > 16384:
+        raise KernelError("rows of up to 16,384 elements")
+    parts = 0
+    if update is not None:
+        parts = _parts_of(update, total_rows, width, "update")
+    elif out is None:
+        raise KernelError("nothing to do: neither an update nor an output")
+    for name, t, shape in (("mix", mix, (count, count)), ("share", share, (count,)), ("read", read, (count,)),
+                           ("weight", weight, (width,)), ("bias", bias, (width,))):
+        if t is not None:
+            _gpu(t, name, torch.float32)
+            if tuple(t.shape) != shape:
+                raise KernelError(f"{name} must be {shape}, got {tuple(t.shape)}")
+    n_rows = total_rows
+    if rows is not None:
+        _gpu(rows, "rows", torch.int32)
+        n_rows = rows.numel()
+        if store and update is not None:
+            raise KernelError("store with a row list is not allowed (rows may repeat)")
+    if out is not None:
+        _gpu(out, "out")
+        if out.shape != (n_rows, width) or weight is None or not eps > 0.0:
+            raise KernelError(f"out must be [{n_rows}, {width}] and come with a weight and a positive eps")
+    _call("hyper", "fe_hyper_norm", _ptr(streams), c_longlong(total_rows * width), c_int(count), _ptr(update), c_int(parts),
+          c_longlong(total_rows * width), _ptr(mix), _ptr(share), _ptr(read), _ptr(weight), _ptr(bias), c_float(eps),
+          c_int(1 if rms else 0), _ptr(out), c_int(_code(out.dtype) if out is not None else FE_F32), _ptr(rows),
+          c_int(n_rows), c_int(width), c_int(1 if (store and update is not None) else 0), _stream())
+    return out
+
+
+def embed_token_pairs(ids: Tensor, table: Tensor, pair_table: Tensor, positions: Tensor, token_seq: Tensor, cu_q: Tensor,
+                      state_slots: Tensor, previous: Tensor, out: Tensor, *, num_seqs: int, buckets: int, mul_prev: int,
+                      mul_cur: int) -> Tensor:
+    """out[t] = float32(table[ids[t]]) + float32(pair_table[r]) with r = (prev * mul_prev + ids[t] * mul_cur)
+    mod buckets, prev the token before t in its sequence: the row before within the step, or, for a
+    sequence's first token of the step, what ``previous`` [slots, 1] (int32) keeps for its slot; a token at
+    position 0 takes row ``buckets`` (the table's last).  Afterwards ``previous`` holds every
+    sequence's last token."""
+    for name, t in (("ids", ids), ("positions", positions), ("token_seq", token_seq), ("previous", previous)):
+        _gpu(t, name, torch.int32)
+    _sequences(cu_q, state_slots, num_seqs)
+    _gpu(table, "table")
+    _gpu(pair_table, "pair_table", table.dtype)
+    _gpu(out, "out", torch.float32)
+    tokens = ids.numel()
+    vocab, hidden = table.shape
+    if pair_table.shape != (buckets + 1, hidden) or buckets < 1 or mul_prev < 0 or mul_cur < 0:
+        raise KernelError(f"pair_table must be [{buckets + 1}, {hidden}], got {tuple(pair_table.shape)}")
+    if out.shape != (tokens, hidden) or positions.numel() != tokens or token_seq.numel() != tokens:
+        raise KernelError("out must be [T, hidden]; positions and token_seq hold one entry per token")
+    if previous.dim() != 2 or previous.shape[1] != 1:
+        raise KernelError("previous must be [slots, 1]")
+    _call("hyper", "fe_embed_token_pairs", _ptr(ids), _ptr(table), _ptr(pair_table), c_int(_code(table.dtype)), _ptr(positions),
+          _ptr(token_seq), _ptr(cu_q), _ptr(state_slots), _ptr(previous), _ptr(out), c_int(tokens), c_int(hidden), c_int(vocab),
+          c_longlong(buckets), c_longlong(mul_prev), c_longlong(mul_cur), c_int(num_seqs), c_int(previous.shape[0]), _stream())
+    return out
+
+
+def scale_rows(x: Tensor, factor: float) -> Tensor:
+    """x *= factor, in place (float32)."""
+    _gpu(x, "x", torch.float32)
+    _call("hyper", "fe_scale_rows", _ptr(x), c_float(factor), c_longlong(x.numel()), _stream())
+    return x
+
+
+# ------------------------------------------------- a norm over the whole projection, rotation, page write
+
+def whole_norm_rope_write(qkv: Tensor, q_weight: Tensor, k_weight: Tensor | None, inv_freq: Tensor | None, positions: Tensor,
+                          token_seq: Tensor, block_table: Tensor, key_pages: Tensor, value_pages: Tensor, q_out: Tensor, *,
+                          q_heads: int, kv_heads: int, head_dim: int, value_dim: int, rotary_dim: int, eps: float,
+                          magnitude: float = 1.0, write_kv: bool = True) -> None:
+    """q (and k) divided by the root mean square over the whole projection (all heads at once, epsilon
+    inside the root) times a weight of that length; then the first ``rotary_dim`` dims of every head turn
+    (dim i pairs with i + rotary_dim / 2, cosines and sines times ``magnitude``); q into ``q_out``
+    [T, Hq * D], k and v into their pages (values transposed).  qkv [T, >= q | k | v] with any row stride;
+    with ``write_kv`` False it holds q alone and the pages are left as they are.  float32 inside."""
+    q_size, kv_size, v_size = q_heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
+    need = q_size + (kv_size + v_size if write_kv else 0)
+    _gpu(qkv, "qkv", contiguous=False)
+    tokens = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.shape[1] < need or qkv.stride(1) != 1:
+        raise KernelError(f"qkv must be [T, >= {need}] with unit inner stride")
+    _gpu(q_out, "q_out", qkv.dtype)
+    if q_out.shape != (tokens, q_size):
+        raise KernelError(f"q_out must be [{tokens}, {q_size}]")
+    _gpu(q_weight, "q_weight", torch.float32)
+    if q_weight.shape != (q_size,):
+        raise KernelError(f"q_weight must be [{q_size}]")
+    if rotary_dim:
+        _gpu(inv_freq, "inv_freq", torch.float32)
+        if inv_freq.shape != (rotary_dim // 2,) or rotary_dim % 2 or rotary_dim > head_dim or rotary_dim > 256:
+            raise KernelError(f"inv_freq must be [{rotary_dim // 2}] for an even rotary_dim <= head_dim and <= 256")
+    _gpu(positions, "positions", torch.int32)
+    _gpu(token_seq, "token_seq", torch.int32)
+    if positions.numel() != tokens or token_seq.numel() != tokens:
+        raise KernelError("positions and token_seq must have one entry per token")
+    block_size = num_blocks = table_stride = 0
+    if write_kv:
+        _gpu(k_weight, "k_weight", torch.float32)
+        if k_weight.shape != (kv_size,):
+            raise KernelError(f"k_weight must be [{kv_size}]")
+        _gpu(block_table, "block_table", torch.int32)
+        _gpu(key_pages, "key_pages", qkv.dtype)
+        _gpu(value_pages, "value_pages", qkv.dtype)
+        if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
+            raise KernelError(f"key pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
+        num_blocks, _, block_size, _ = key_pages.shape
+        if value_pages.shape != (num_blocks, kv_heads, value_dim, block_size):
+            raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {value_dim}, block_size], got {tuple(value_pages.shape)}")
+        if block_table.dim() != 2 or block_table.stride(1) != 1:
+            raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+        table_stride = block_table.stride(0)
+    if not eps > 0.0:
+        raise KernelError("eps must be positive")
+    stride = qkv.stride(0) if tokens > 1 else max(qkv.stride(0), qkv.shape[1])
+    _call("whole_norm_rope", "fe_whole_norm_rope_write", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(q_weight),
+          _ptr(k_weight if write_kv else None), _ptr(inv_freq if rotary_dim else None), _ptr(positions), _ptr(token_seq),
+          _ptr(block_table if write_kv else None), c_int(table_stride), _ptr(key_pages if write_kv else None),
+          _ptr(value_pages if write_kv else None), _ptr(q_out), c_int(tokens), c_int(q_heads), c_int(kv_heads), c_int(head_dim),
+          c_int(value_dim), c_int(rotary_dim), c_float(eps), c_float(magnitude), c_int(1 if write_kv else 0), c_int(block_size),
+          c_int(num_blocks), _stream())
+
+
+# ------------------------------------------------- a mixture of experts
+
+def moe_route(x: Tensor, router_weight: Tensor, router_bias: Tensor | None, top: int) -> tuple[Tensor, Tensor]:
+    """Router logits ``x W^T + b`` in float32; for every token the ``top`` experts with the largest logits
+    (int32 [T, top], largest first, the lowest index among equals) and the softmax over their logits alone
+    (float32 [T, top])."""
+    _gpu(x, "x")
+    _gpu(router_weight, "router_weight", x.dtype)
+    tokens, hidden = x.shape
+    experts = router_weight.shape[0]
+    if router_weight.shape != (experts, hidden) or not 1 <= top <= min(experts, 16) or experts > 1024:
+        raise KernelError(f"router_weight must be [experts <= 1024, {hidden}] and top between 1 and min(experts, 16)")
+    if router_bias is not None:
+        _gpu(router_bias, "router_bias", torch.float32)
+        if router_bias.shape != (experts,):
+            raise KernelError(f"router_bias must be [{experts}]")
+    chosen = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
+    _call("moe", "fe_moe_route", _ptr(x), _ptr(router_weight), c_int(_code(x.dtype)), _ptr(router_bias), _ptr(chosen),
+          _ptr(weights), c_int(tokens), c_int(hidden), c_int(experts), c_int(top), _stream())
+    return chosen, weights
+
+
+def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, down: Tensor, out: Tensor, *, limit: float,
+                alpha: float) -> Tensor:
+    """out[k, t] = weights[t, k] * down[e] @ act, e = chosen[t, k], with ``act = min(g, limit) *
+    sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)``, ``g = gate_up[e, :F] @ x[t]``,
+    ``u = gate_up[e, F:] @ x[t]``.  x [T, H]; gate_up [E, 2F, H]; down [E, H, F]; out float32 [top, T, H]
+    (one part per choice).  The pairs are sorted by expert on the device and two grouped products run
+    over the sorted rows."""
+    _gpu(x, "x")
+    _gpu(chosen, "chosen", torch.int32)
+    _gpu(weights, "weights", torch.float32)
+    _gpu(gate_up, "gate_up", x.dtype)
+    _gpu(down, "down", x.dtype)
+    _gpu(out, "out", torch.float32)
+    tokens, hidden = x.shape
+    top = chosen.shape[1] if chosen.dim() == 2 else 0
+    if gate_up.dim() != 3 or gate_up.shape[2] != hidden or gate_up.shape[1] % 2:
+        raise KernelError(f"gate_up must be [experts, 2F, {hidden}], got {tuple(gate_up.shape)}")
+    experts, inner = gate_up.shape[0], gate_up.shape[1] // 2
+    if down.shape != (experts, hidden, inner):
+        raise KernelError(f"down must be [{experts}, {hidden}, {inner}], got {tuple(down.shape)}")
+    if chosen.shape != (tokens, top) or weights.shape != (tokens, top) or not 1 <= top <= 16 or experts > 1024:
+        raise KernelError("chosen and weights must be [T, top <= 16] and experts at most 1,024")
+    if out.shape != (top, tokens, hidden):
+        raise KernelError(f"out must be [{top}, {tokens}, {hidden}], got {tuple(out.shape)}")
+    if not limit > 0.0:
+        raise KernelError("limit must be positive")
+    pairs = tokens * top
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=x.device)
+    order = torch.empty(pairs, dtype=torch.int32, device=x.device)
+    act = torch.empty((pairs, inner), dtype=x.dtype, device=x.device)
+    code = c_int(_code(x.dtype))
+    _call("moe", "fe_moe_plan", _ptr(chosen), c_int(pairs), c_int(experts), _ptr(offsets), _ptr(order), _stream())
+    _call("moe", "fe_moe_gate_up", _ptr(x), _ptr(gate_up), code, _ptr(offsets), _ptr(order), _ptr(act), c_int(tokens), c_int(top),
+          c_int(experts), c_int(hidden), c_int(inner), c_float(limit), c_float(alpha), _stream())
+    _call("moe", "fe_moe_down", _ptr(act), _ptr(down), code, _ptr(offsets), _ptr(order), _ptr(weights), _ptr(out), c_int(tokens),
+          c_int(top), c_int(experts), c_int(hidden), c_int(inner), _stream())
+    return out
+
+
+def linear_gated(x: Tensor, gate_up_weight: Tensor, *, limit: float, alpha: float) -> Tensor:
+    """``min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)`` with g and u the two
+    halves of ``x @ gate_up_weight^T`` ([2F, H]: gate rows first); the result [T, F] in x's dtype."""
+    gate_up = linear(x, gate_up_weight)
+    tokens, width = gate_up.shape
+    if width % 2 or not limit > 0.0:
+        raise KernelError("a gated weight needs an even number of rows and a positive limit")
+    out = torch.empty((tokens, width // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _call("moe", "fe_gated_act", _ptr(gate_up), _ptr(out), c_int(_code(gate_up.dtype)), c_int(tokens), c_int(width // 2),
+          c_float(limit), c_float(alpha), _stream())
     return out

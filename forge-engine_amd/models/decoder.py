@@ -94,11 +94,16 @@ class DecoderModel:
         """One entry per schedule call (what its mixer asks of the cache)."""
         return [self.layers[call.layer].cache_needs() for call in self.schedule]
 
+    def embedding_needs(self) -> CacheNeeds:
+        """Fixed-size state per request that the embedding keeps between steps."""
+        return self.embedding.cache_needs()
+
     # --------------------------------------------------------------- running
-    def forward(self, batch, cache_views: list[CacheView | None]) -> Tensor:
+    def forward(self, batch, cache_views: list[CacheView | None], embedding_view: CacheView | None = None) -> Tensor:
         """Run the step's tokens through every scheduled layer; float32 logits
-        [len(batch.want_rows), vocab] at the wanted rows."""
-        residual = self.embedding.forward(batch)
+        [len(batch.want_rows), vocab] at the wanted rows.  ``embedding_view``: the states of an
+        embedding that keeps some."""
+        residual = self.embedding.forward(batch) if embedding_view is None else self.embedding.forward(batch, embedding_view)
         for index, call in enumerate(self.schedule):
             self.layers[call.layer].forward(residual, batch, cache_views[index], call.writes_cache)
         if batch.num_wanted == 0:

@@ -16,8 +16,13 @@ as fixed-size state); ``unit_norm_eps`` (after the rotation, q and k heads are d
 root mean square, no weight); ``chunk`` (token i sees key j <= i only if both lie in the same
 run of ``chunk`` positions counted from position 0); ``sink`` (a learned number per query head
 whose exponential joins the softmax's denominator, without key or value); ``output_gate``
-(the concatenated heads times sigmoid(W_g x) before the output projection); ``names`` (what the
-tensors are called in the checkpoint).  With any of them the step takes the general path:
+(the concatenated heads times sigmoid(W_g x) before the output projection; with ``head_gate`` W_g has
+one row per query head and the whole head is multiplied by that one number); ``whole_norm_eps``
+(q, and k, divided by the root mean square over the whole projection, all heads at once, times a
+weight of that size, before the rotation); ``softcap`` (scores, after the scale, bounded as
+``cap * tanh(score / cap)``); ``own_kv`` False (the layer has no k and v tensors at all and is only
+ever scheduled to read another call's cache); ``names`` (what the tensors are called in the
+checkpoint).  A position part may scale its cosines and sines (``magnitude``).  With any of them the step takes the general path:
 one product for q, k, v (and the gate), one kernel for convolution, rotation, norms and the
 page write, the masked attention kernel, the gate, the output projection.
 """
@@ -40,7 +45,8 @@ class GroupedQueryAttention(Mixer):
                  bias: bool = False, window: int | None = None, scale: float | None = None,
                  value_dim: int | None = None, conv_taps: int = 0, unit_norm_eps: float | None = None,
                  chunk: int | None = None, sink: bool = False, output_gate: bool = False,
-                 names: dict[str, str] | None = None) -> None:
+                 head_gate: bool = False, whole_norm_eps: float | None = None, softcap: float | None = None,
+                 own_kv: bool = True, names: dict[str, str] | None = None) -> None:
         super().__init__(ctx, prefix)
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
@@ -59,14 +65,24 @@ class GroupedQueryAttention(Mixer):
         self.unit_norm_eps = unit_norm_eps
         self.chunk = chunk
         self.sink = sink
-        self.output_gate = output_gate
+        self.output_gate = output_gate or head_gate
+        self.head_gate = head_gate
+        self.whole_norm_eps = whole_norm_eps
+        self.softcap = None if softcap is None else float(softcap)
+        self.own_kv = own_kv
+        self.gate_size = 0 if not self.output_gate else (num_heads if head_gate else self.out_size)
+        if whole_norm_eps is not None and (self.conv_taps or unit_norm_eps is not None or bias):
+            raise ValueError("a norm over the whole projection is not combined with convolutions, unit norms or biases")
+        if not own_kv and whole_norm_eps is None:
+            raise ValueError("a layer without keys and values of its own takes the path of the whole-projection norm")
         if self.conv_taps < 0:
             raise ValueError("a short convolution has at least one tap (0: none)")
         if chunk is not None and (chunk < 1 or window is not None):
             raise ValueError("chunk must be positive and cannot be combined with a window")
         # the general path: anything the fused kernels of the plain arrangement do not know
         self.general = bool(self.value_dim != head_dim or self.conv_taps or unit_norm_eps is not None
-                            or chunk is not None or sink or output_gate)
+                            or chunk is not None or sink or self.output_gate or whole_norm_eps is not None
+                            or softcap is not None or not own_kv)
         if self.general and qk_norm_eps is not None:
             raise ValueError("weighted q/k norms before the rotation are not combined with the general path's options")
         self.names = dict(self.DEFAULT_NAMES, **(names or {}))
@@ -76,11 +92,14 @@ class GroupedQueryAttention(Mixer):
         self.scale = head_dim ** -0.5 if scale is None else float(scale)
         self.position = build_part("position", position, ctx)
         self.conv_channels = self.q_size + self.kv_size + self.v_size
-        width = self.conv_channels + (self.out_size if output_gate else 0)
-        self._rows = {"q": (0, self.q_size), "k": (self.q_size, self.kv_size),
-                      "v": (self.q_size + self.kv_size, self.v_size)}
-        if output_gate:
-            self._rows["gate"] = (self.conv_channels, self.out_size)
+        if not own_kv:
+            self.conv_channels = self.q_size
+        width = self.conv_channels + self.gate_size
+        self._rows = {"q": (0, self.q_size)}
+        if own_kv:
+            self._rows.update({"k": (self.q_size, self.kv_size), "v": (self.q_size + self.kv_size, self.v_size)})
+        if self.output_gate:
+            self._rows["gate"] = (self.conv_channels, self.gate_size)
         self._width = width
         self.conv_weight: Tensor | None = None
         self.sink_weight: Tensor | None = None
@@ -104,10 +123,15 @@ class GroupedQueryAttention(Mixer):
         n = {key: self.name(leaf) for key, leaf in self.names.items()}
         specs = {
             n["q"]: ParamSpec((self.q_size, self.hidden_size)),
-            n["k"]: ParamSpec((self.kv_size, self.hidden_size)),
-            n["v"]: ParamSpec((self.v_size, self.hidden_size)),
             n["o"]: ParamSpec((self.hidden_size, self.out_size)),
         }
+        if self.own_kv:
+            specs[n["k"]] = ParamSpec((self.kv_size, self.hidden_size))
+            specs[n["v"]] = ParamSpec((self.v_size, self.hidden_size))
+        if self.whole_norm_eps is not None:
+            specs[n["q_norm"]] = ParamSpec((self.q_size,), kind="vector", init="norm")
+            if self.own_kv:
+                specs[n["k_norm"]] = ParamSpec((self.kv_size,), kind="vector", init="norm")
         if self.bias:
             specs[n["q_bias"]] = ParamSpec((self.q_size,), kind="vector", init="zeros")
             specs[n["k_bias"]] = ParamSpec((self.kv_size,), kind="vector", init="zeros")
@@ -123,7 +147,7 @@ class GroupedQueryAttention(Mixer):
         if self.sink:
             specs[n["sink"]] = ParamSpec((self.num_heads,), kind="vector", init="unit")
         if self.output_gate:
-            specs[n["gate"]] = ParamSpec((self.out_size, self.hidden_size))
+            specs[n["gate"]] = ParamSpec((self.gate_size, self.hidden_size))
         return specs
 
     def set_param(self, name: str, tensor: Tensor) -> None:
@@ -228,16 +252,22 @@ class GroupedQueryAttention(Mixer):
 
     def _forward_general(self, x: Tensor, batch, cache: CacheView, writes_cache: bool, stream, inv_freq,
                          rotary_dim: int) -> Tensor | None:
-        if not writes_cache:
-            raise ValueError("the general attention path writes its own keys and values")
+        if writes_cache != self.own_kv or (not writes_cache and self.whole_norm_eps is None):
+            raise ValueError("the general attention path writes its own keys and values, except for a layer that "
+                             "has none and reads another call's")
         qkv = ops.linear(x, self.qkv_weight)        # [T, q | k | v (| gate)]; the bias is added by the kernel below
         q = torch.empty((x.shape[0], self.q_size), dtype=x.dtype, device=x.device)
-        ops.conv_rope_norm_write(
-            qkv, self.conv_bias, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps > 1 else None, inv_freq,
-            batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
-            cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
-            kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,
-            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps, taps=self.conv_taps)
+        magnitude = self.position.magnitude()
+        if self.whole_norm_eps is not None:
+            ops.whole_norm_rope_write(
+                qkv, self.q_norm, self.k_norm, inv_freq, batch.positions, batch.token_seq, cache.block_table,
+                cache.key_pages, cache.value_pages, q, q_heads=self.num_heads, kv_heads=self.num_kv_heads,
+                head_dim=self.head_dim, value_dim=self.value_dim, rotary_dim=rotary_dim, eps=self.whole_norm_eps,
+                magnitude=magnitude, write_kv=writes_cache)
+        elif magnitude != 1.0:
+            raise ValueError("scaled cosines and sines come with the whole-projection norm's kernel only")
+        else:
+            self._conv_rope(qkv, q, batch, cache, inv_freq, rotary_dim)
         attn = torch.empty((x.shape[0], self.out_size), dtype=x.dtype, device=x.device)
         ops.masked_attention(
             q, cache.key_pages, cache.value_pages, attn, batch.cu_q, batch.ctx_len, cache.block_table,
@@ -245,9 +275,17 @@ class GroupedQueryAttention(Mixer):
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim, scale=self.scale,
             window=self.window, chunk=self.chunk, sink=self.sink_weight,
             gate=qkv[:, self.conv_channels:] if self.output_gate else None, num_decode=batch.num_decode,
-            max_ctx=batch.max_ctx)
+            max_ctx=batch.max_ctx, softcap=self.softcap, head_gate=self.head_gate)
         update = ops.linear_update(attn, self.o_weight)
         return update if self.o_bias_f32 is None else ops.add_bias(update, self.o_bias_f32)
+
+    def _conv_rope(self, qkv: Tensor, q: Tensor, batch, cache: CacheView, inv_freq, rotary_dim: int) -> None:
+        ops.conv_rope_norm_write(
+            qkv, self.conv_bias, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps > 1 else None, inv_freq,
+            batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
+            cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
+            kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,
+            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps, taps=self.conv_taps)
 
     def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
         """Every sequence of the step brings one token, and the sizes are ones that the
@@ -262,7 +300,7 @@ class GroupedQueryAttention(Mixer):
 
     def kernel_libraries(self):
         if self.general:
-            return {"conv_rope", "attention_masked", "attention_decode", "attention_prefill", "stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+            return {"whole_norm_rope" if self.whole_norm_eps is not None else "conv_rope", "attention_masked", "attention_decode", "attention_prefill", "stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
         return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 
 

@@ -33,7 +33,8 @@ class ParamSpec:
     biases, widened to float32, which is exact), ``int_table`` (int32).
     ``init``: how the random-weights mode draws it: ``normal`` N(0, 0.02),
     ``norm`` 1 + N(0, 0.05), ``zeros``, ``unit`` N(0, 0.25), ``uniform`` U(0, 1), ``taps`` (a short
-    convolution: N(0, 0.04) with one added to the newest tap).
+    convolution: N(0, 0.04) with one added to the newest tap), ``small`` N(0, 0.01), ``router``
+    N(0, 0.25), ``identity`` (the identity plus N(0, 0.01)).
     """
 
     shape: tuple[int, ...]
@@ -50,25 +51,60 @@ class BuildContext:
 
 class Residual:
     """The float32 residual stream of one step with at most one update that has
-    not been added yet, so that the add can be fused into the next norm."""
+    not been added yet, so that the add can be fused into the next norm.
+
+    A design with several residual streams keeps them in ``streams`` [S, T, W] (``h`` is then only
+    where their sum is put at the end): an arrangement widens the one stream of the embedding into
+    S copies (``widen``), its pending update comes with the matrix that mixes the old streams into
+    the new ones and each stream's share of the update (``add_mixed``), and a norm that reads
+    streams (``reads_streams``) takes their sum, or any weighted sum, as its input: the last norm
+    of such a model reads the plain sum."""
 
     def __init__(self, h: Tensor) -> None:
         self.h = h
         self.pending: Tensor | None = None
+        self.streams: Tensor | None = None
+        self.pending_mix: tuple[Tensor, Tensor] | None = None    # (mix [S, S] indexed [from, to], share [S])
 
     def add(self, update: Tensor | None) -> None:
         """Leave an update pending; None: the part has added it into the stream itself."""
         self.flush()
         self.pending = update
 
+    def add_mixed(self, update: Tensor, mix: Tensor, share: Tensor) -> None:
+        """Several streams: leave ``x_t <- sum_s mix[s, t] x_s + share[t] * update`` pending."""
+        self.flush()
+        self.pending, self.pending_mix = update, (mix, share)
+
+    def take_pending(self):
+        """(update, mix, share) of what is pending, which the caller now applies itself."""
+        update, mixed = self.pending, self.pending_mix
+        self.pending = self.pending_mix = None
+        return (update, *(mixed or (None, None)))
+
+    def widen(self, count: int) -> Tensor:
+        """The streams [count, T, W]: at first ``count`` copies of the one stream."""
+        if self.streams is None:
+            self.flush()
+            self.streams = self.h.unsqueeze(0).repeat(count, 1, 1)
+        elif self.streams.shape[0] != count:
+            raise ValueError(f"the model's layers disagree on the number of streams ({self.streams.shape[0]} and {count})")
+        return self.streams
+
     def open(self) -> Tensor:
         """The stream with nothing pending, for a part that adds its update itself."""
+        if self.streams is not None:
+            raise ValueError("a part that adds into the stream itself needs a model with one stream")
         return self.flush()
 
     def flush(self) -> Tensor:
         if self.pending is not None:
-            ops.add_rows(self.h, self.pending)
-            self.pending = None
+            if self.streams is not None:
+                update, mix, share = self.take_pending()
+                ops.hyper_norm(self.streams, update, mix, share, None, None, None, 0.0, None)
+            else:
+                ops.add_rows(self.h, self.pending)
+                self.pending = None
         return self.h
 
 
@@ -116,7 +152,12 @@ class Part:
 class Embedding(Part):
     role = "embedding"
 
-    def forward(self, batch) -> Residual:
+    def cache_needs(self) -> CacheNeeds:
+        """Fixed-size state per request that the embedding keeps between steps (none by default);
+        an embedding that asks for some gets ``cache=`` (a ``CacheView`` with its states)."""
+        return CacheNeeds()
+
+    def forward(self, batch, cache: CacheView | None = None) -> Residual:
         raise NotImplementedError
 
 
@@ -136,6 +177,10 @@ class PositionEncoding(Part):
         """(inv_freq float32 [rotary_dim / 2], rotary_dim) for mixers that rotate
         q and k, or None."""
         return None
+
+    def magnitude(self) -> float:
+        """A factor on every cosine and sine of the rotation (1: a plain rotation)."""
+        return 1.0
 
 
 class Mixer(Part):

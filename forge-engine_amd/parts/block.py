@@ -26,6 +26,8 @@ class PreNormBlock(Block):
             residual.add(self.mixer.forward(x, batch, cache, writes_cache, stream=residual.open()))
         else:
             residual.add(self.mixer.forward(x, batch, cache, writes_cache))
+        if self.feed_forward is None:
+            return
         y = self.norms["post_mixer"].forward(residual)
         if self.feed_forward.takes_stream:
             residual.add(self.feed_forward.forward(y, batch, stream=residual.open()))
@@ -92,5 +94,65 @@ class OutputNormBlock(Block):
         return {"stream_ops"}
 
 
+class HyperConnectionBlock(Block):
+    """Pre-norm sublayers over ``streams`` residual streams instead of one.  Sublayer q (the mixer,
+    then the feed-forward) reads ``u = sum_s in_q[s] x_s``, computes ``y = sublayer(norm_q(u))``, and
+    every stream is replaced at once, from the old ones, by ``x_t = sum_s mix_q[s, t] x_s +
+    out_q[t] y``.  The tensors ``in`` [S], ``out`` [S] and ``mix`` [S, S] (indexed [from, to]) live
+    under ``<prefix>.<hc1 | hc2>``.  The streams start as copies of the embedding's output and the
+    model's last norm reads their sum.  The update is left pending on the stream with its matrix
+    and applied inside the next norm's kernel, which forms the next sublayer's input in the same
+    pass.  A layer may have no feed-forward."""
+
+    NORMS = ("input", "post_mixer")
+    SUBLAYERS = ("hc1", "hc2")
+
+    def __init__(self, ctx: BuildContext, mixer, feed_forward, norms, prefix: str = "", *, streams: int,
+                 names: dict[str, str] | None = None) -> None:
+        super().__init__(ctx, mixer, feed_forward, norms, prefix)
+        if not 1 <= streams <= 8:
+            raise ValueError(f"one to eight residual streams, not {streams}")
+        for role, norm in norms.items():
+            if not getattr(norm, "reads_streams", False):
+                raise ValueError(f"the norm '{role}' of a layer with several streams must be one that reads streams")
+        self.streams = streams
+        self.names = dict({"in": "in", "out": "out", "mix": "mix"}, **(names or {}))
+        self.sublayers = self.SUBLAYERS if feed_forward is not None else self.SUBLAYERS[:1]
+        self.weights: dict[str, Tensor] = {}
+
+    def _name(self, sublayer: str, key: str) -> str:
+        return self.name(f"{sublayer}.{self.names[key]}")
+
+    def param_specs(self):
+        s = self.streams
+        specs = {}
+        for sublayer in self.sublayers:
+            specs[self._name(sublayer, "in")] = ParamSpec((s,), kind="vector", init="uniform")
+            specs[self._name(sublayer, "out")] = ParamSpec((s,), kind="vector", init="norm")
+            specs[self._name(sublayer, "mix")] = ParamSpec((s, s), kind="vector", init="identity")
+        return specs
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        for sublayer in self.sublayers:
+            for key in ("in", "out", "mix"):
+                if name == self._name(sublayer, key):
+                    self.weights[f"{sublayer}.{key}"] = tensor.contiguous()
+                    return
+        raise KeyError(name)
+
+    def forward(self, residual: Residual, batch, cache: CacheView | None, writes_cache: bool = True) -> None:
+        residual.widen(self.streams)
+        w = self.weights
+        x = self.norms["input"].forward(residual, read=w["hc1.in"])
+        residual.add_mixed(self.mixer.forward(x, batch, cache, writes_cache), w["hc1.mix"], w["hc1.out"])
+        if self.feed_forward is not None:
+            y = self.norms["post_mixer"].forward(residual, read=w["hc2.in"])
+            residual.add_mixed(self.feed_forward.forward(y, batch), w["hc2.mix"], w["hc2.out"])
+
+    def kernel_libraries(self):
+        return {"hyper"}
+
+
+register_part("block", "hyper_connections", HyperConnectionBlock)
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "output_norm", OutputNormBlock)

@@ -13,6 +13,7 @@ from torch import Tensor
 
 from ..kernels import ops
 from ..registry import register_part
+from ..cache.spec import CacheNeeds, CacheView, FixedState
 from .base import BuildContext, Embedding, Head, ParamSpec, Residual
 
 
@@ -42,10 +43,51 @@ class TokenEmbedding(Embedding):
         return {"rowwise"}
 
 
+class TokenPairEmbedding(TokenEmbedding):
+    """The token's row plus a row of a second table chosen by the token and the one before it:
+    row ``(prev * mul_prev + cur * mul_cur) mod buckets``, and for a sequence's first token the
+    table's last row (number ``buckets``).  The previous token is fixed-size state of the request
+    (one integer a slot), so a request may be cut into steps anywhere."""
+
+    PREVIOUS = "previous_token"
+
+    def __init__(self, ctx: BuildContext, prefix: str, *, vocab_size: int, hidden_size: int, buckets: int,
+                 mul_prev: int, mul_cur: int, leaf: str = "weight", pair_name: str = "pairs") -> None:
+        """``pair_name``: the second table's full name in the checkpoint."""
+        super().__init__(ctx, prefix, vocab_size=vocab_size, hidden_size=hidden_size, leaf=leaf)
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.pair_name = pair_name
+        self.pair_weight: Tensor | None = None
+
+    def param_specs(self):
+        return dict(super().param_specs(), **{self.pair_name: ParamSpec((self.buckets + 1, self.hidden_size))})
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        if name == self.pair_name:
+            self.pair_weight = tensor
+        else:
+            super().set_param(name, tensor)
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(state={self.PREVIOUS: FixedState((1,), torch.int32)})
+
+    def forward(self, batch, cache: CacheView | None = None) -> Residual:
+        h = torch.empty((batch.num_tokens, self.hidden_size), dtype=torch.float32, device=self.weight.device)
+        ops.embed_token_pairs(batch.token_ids, self.weight, self.pair_weight, batch.positions, batch.token_seq, batch.cu_q,
+                              batch.state_slots, cache.states[self.PREVIOUS], h, num_seqs=batch.num_seqs,
+                              buckets=self.buckets, mul_prev=self.mul_prev, mul_cur=self.mul_cur)
+        return Residual(h)
+
+    def kernel_libraries(self):
+        return {"rowwise", "hyper"}
+
+
 class LMHead(Head):
     def __init__(self, ctx: BuildContext, prefix: str, *, vocab_size: int, hidden_size: int,
-                 tied: bool = False, leaf: str = "weight") -> None:
+                 tied: bool = False, leaf: str = "weight", scale: float = 1.0) -> None:
+        """``scale``: a factor on the logits."""
         super().__init__(ctx, prefix)
+        self.scale = float(scale)
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied = tied
@@ -71,11 +113,13 @@ class LMHead(Head):
 
     def forward(self, z: Tensor) -> Tensor:
         # float32 accumulation and float32 logits in both modes (no rounding of the logits)
-        return ops.linear(z, self.matrix(), out_dtype=torch.float32)
+        logits = ops.linear(z, self.matrix(), out_dtype=torch.float32)
+        return logits if self.scale == 1.0 else ops.scale_rows(logits, self.scale)
 
     def kernel_libraries(self):
-        return {"gemm_f32", "gemm_skinny"}
+        return {"gemm_f32", "gemm_skinny"} | ({"hyper"} if self.scale != 1.0 else set())
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("embedding", "token_pair_embedding", TokenPairEmbedding)
 register_part("head", "lm_head", LMHead)

@@ -1,0 +1,130 @@
+"""A mixture of small gated feed-forward layers chosen per token by a router.
+
+Router: ``z = W_r x + b_r`` in float32; the ``top`` experts with the largest logits are chosen and
+their weights are the softmax over the chosen logits alone.  Expert (no biases):
+``g = min(W_gate x, limit)``, ``u = clamp(W_up x, -limit, limit)``,
+``y = W_down (g * sigmoid(alpha g) * (u + 1))``.  The output is the weighted sum of the chosen
+experts' outputs, plus a shared expert of the same form (sizes and limit of its own) that every
+token takes.
+
+A step sorts its (token, choice) pairs by expert on the device and runs two grouped products over
+the sorted rows (gate and up with the activation as their ending, then down, weighted by the
+router); nothing is decided on the host, so steps are captured like any other.  The update comes
+back in parts, one per choice and the shared expert's behind them, which the next norm adds up in
+that order: a token's sum does not depend on what else is in the step.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from ..kernels import ops
+from ..registry import register_part
+from .base import BuildContext, FeedForward, ParamSpec
+
+
+class RoutedExperts(FeedForward):
+    def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, experts: int, top: int,
+                 intermediate_size: int, limit: float, alpha: float = 1.702, shared_size: int | None = None,
+                 shared_limit: float | None = None, names: dict[str, str] | None = None) -> None:
+        """``names``: what the tensors are called behind the prefix; ``expert`` is a pattern with
+        ``{e}`` for the expert's number."""
+        super().__init__(ctx, prefix)
+        if not 1 <= top <= experts:
+            raise ValueError(f"a token takes between one and all {experts} experts, not {top}")
+        if top > 16 or experts > 1024:
+            raise ValueError("up to 16 experts a token out of up to 1,024")
+        self.hidden_size = hidden_size
+        self.experts, self.top = experts, top
+        self.intermediate_size = intermediate_size
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.shared_size = shared_size
+        self.shared_limit = float(limit if shared_limit is None else shared_limit)
+        self.names = dict({"expert": "experts.{e}", "shared": "shared", "router": "router.weight", "router_bias": "router.bias",
+                           "gate": "gate", "up": "up", "down": "down"}, **(names or {}))
+        self.router_weight: Tensor | None = None
+        self.router_bias: Tensor | None = None
+        self.gate_up: Tensor | None = None          # [experts, 2 F, H]: an expert's gate rows, then its up rows
+        self.down: Tensor | None = None             # [experts, H, F]
+        self.shared_gate_up: Tensor | None = None   # [2 Fs, H]
+        self.shared_down: Tensor | None = None
+
+    def _expert_name(self, expert: int | None, which: str) -> str:
+        owner = self.names["shared"] if expert is None else self.names["expert"].format(e=expert)
+        return self.name(f"{owner}.{self.names[which]}")
+
+    def param_specs(self):
+        f, h = self.intermediate_size, self.hidden_size
+        specs = {self.name(self.names["router"]): ParamSpec((self.experts, h), init="router"),
+                 self.name(self.names["router_bias"]): ParamSpec((self.experts,), kind="vector", init="small")}
+        for expert in range(self.experts):
+            specs[self._expert_name(expert, "gate")] = ParamSpec((f, h))
+            specs[self._expert_name(expert, "up")] = ParamSpec((f, h))
+            specs[self._expert_name(expert, "down")] = ParamSpec((h, f))
+        if self.shared_size:
+            specs[self._expert_name(None, "gate")] = ParamSpec((self.shared_size, h))
+            specs[self._expert_name(None, "up")] = ParamSpec((self.shared_size, h))
+            specs[self._expert_name(None, "down")] = ParamSpec((h, self.shared_size))
+        self._owners = {}
+        for expert in [*range(self.experts), None] if self.shared_size else range(self.experts):
+            for which in ("gate", "up", "down"):
+                self._owners[self._expert_name(expert, which)] = (expert, which)
+        return specs
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        f, h = self.intermediate_size, self.hidden_size
+        if name == self.name(self.names["router"]):
+            self.router_weight = tensor.contiguous()
+            return
+        if name == self.name(self.names["router_bias"]):
+            self.router_bias = tensor.contiguous()
+            return
+        if not hasattr(self, "_owners"):
+            self.param_specs()
+        if name not in self._owners:
+            raise KeyError(name)
+        expert, which = self._owners[name]
+        if expert is None:
+            if which == "down":
+                self.shared_down = tensor
+                return
+            if self.shared_gate_up is None:
+                self.shared_gate_up = torch.empty((2 * self.shared_size, h), dtype=tensor.dtype, device=tensor.device)
+            start = 0 if which == "gate" else self.shared_size
+            self.shared_gate_up[start:start + self.shared_size].copy_(tensor)
+            return
+        if which == "down":
+            if self.down is None:
+                self.down = torch.empty((self.experts, h, f), dtype=tensor.dtype, device=tensor.device)
+            self.down[expert].copy_(tensor)
+            return
+        if self.gate_up is None:
+            self.gate_up = torch.empty((self.experts, 2 * f, h), dtype=tensor.dtype, device=tensor.device)
+        start = 0 if which == "gate" else f
+        self.gate_up[expert, start:start + f].copy_(tensor)
+
+    def finalize(self) -> None:
+        if self.gate_up.dtype != self.down.dtype or self.gate_up.dtype != self.router_weight.dtype:
+            raise ValueError(f"{self.prefix}: the experts' matrices and the router must be stored in one dtype")
+
+    def forward(self, x: Tensor, batch=None) -> Tensor:
+        tokens = x.shape[0]
+        chosen, weights = ops.moe_route(x, self.router_weight, self.router_bias, self.top)
+        parts = self.top + (1 if self.shared_size else 0)
+        update = torch.empty((parts, tokens, self.hidden_size), dtype=torch.float32, device=x.device)
+        ops.moe_experts(x, chosen, weights, self.gate_up, self.down, update[:self.top], limit=self.limit, alpha=self.alpha)
+        if self.shared_size:
+            act = ops.linear_gated(x, self.shared_gate_up, limit=self.shared_limit, alpha=self.alpha)
+            shared = ops.linear_update(act, self.shared_down)
+            if shared.dim() == 2:
+                update[self.top].copy_(shared)
+            else:           # the product came in parts of K itself
+                update = torch.cat([update[:self.top], shared])
+        return update
+
+    def kernel_libraries(self):
+        return {"moe", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)

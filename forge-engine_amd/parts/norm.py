@@ -65,5 +65,51 @@ class UpdateRMSNorm(RMSNorm):
         return {"rowwise", "stream_ops"}
 
 
+class LayerNorm(Norm):
+    """``(x - mean) / sqrt(variance + eps) * w + b`` over a row, the variance being the mean of the
+    squared deviations; float32 inside, fused with the add of the pending update like the other
+    norms.  It also serves models with several residual streams (``reads_streams``): its input is
+    then ``sum_s read[s] x_s`` (``read`` None: the plain sum), taken after the pending update went
+    into the streams through its mixing matrix, all in the same kernel."""
+
+    reads_streams = True
+
+    def __init__(self, ctx: BuildContext, prefix: str, *, size: int, eps: float, leaf: str = "weight",
+                 bias_leaf: str = "bias") -> None:
+        """``leaf`` / ``bias_leaf``: the tensors' names behind the prefix ("": the prefix itself)."""
+        super().__init__(ctx, prefix)
+        self.size = size
+        self.eps = float(eps)
+        self.leaf, self.bias_leaf = leaf, bias_leaf
+        self.weight: Tensor | None = None
+        self.bias: Tensor | None = None
+
+    def param_specs(self):
+        return {self.name(self.leaf): ParamSpec((self.size,), kind="vector", init="norm"),
+                self.name(self.bias_leaf): ParamSpec((self.size,), kind="vector", init="small")}
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        if name == self.name(self.leaf):
+            self.weight = tensor
+        elif name == self.name(self.bias_leaf):
+            self.bias = tensor
+        else:
+            raise KeyError(name)
+
+    def forward(self, residual: Residual, rows: Tensor | None = None, read: Tensor | None = None) -> Tensor:
+        streams = residual.streams if residual.streams is not None else residual.h.unsqueeze(0)
+        count = streams.shape[1] if rows is None else rows.numel()
+        out = torch.empty((count, self.size), dtype=self.ctx.dtype, device=streams.device)
+        if rows is not None:     # the chosen rows alone; stream and pending update are left as they are
+            update, mixed = residual.pending, residual.pending_mix or (None, None)
+            return ops.hyper_norm(streams, update, *mixed, read, self.weight, self.bias, self.eps, out, rows=rows, store=False)
+        update, mix, share = residual.take_pending()
+        return ops.hyper_norm(streams, update, mix, share, read, self.weight, self.bias, self.eps, out)
+
+    def kernel_libraries(self):
+        return {"hyper"}
+
+
+register_part("norm", "layer_norm", LayerNorm)
 register_part("norm", "rms_norm", RMSNorm)
 register_part("norm", "rms_norm_of_update", UpdateRMSNorm)

@@ -74,4 +74,4 @@ def _load_builtin() -> None:
         return
     _BUILTIN_LOADED = True
     from . import parts  # noqa: F401  registers the built-in parts
-    from .models import mazanex, qwen3  # noqa: F401  register Mazanex and Qwen3ForCausalLM
+    from .models import mazanex, qwen3, rekezen  # noqa: F401  register Mazanex, Qwen3ForCausalLM and Rekezen

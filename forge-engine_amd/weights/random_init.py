@@ -34,6 +34,12 @@ def _draw(spec: ParamSpec, generator: torch.Generator, device) -> torch.Tensor:
         return noise * 0.5
     if spec.init == "uniform":     # blend weights between a token and the one before it
         return torch.rand(spec.shape, generator=generator, dtype=torch.float32, device=device)
+    if spec.init == "small":       # biases: small, but not zero, so that leaving one out shows
+        return noise * 0.1
+    if spec.init == "router":      # routers: logits far enough apart that roundings do not change the choice
+        return noise * 0.5
+    if spec.init == "identity":    # square matrices that mix streams: near the identity
+        return torch.eye(spec.shape[-1], dtype=torch.float32, device=device).expand(spec.shape) + noise * 0.1
     if spec.init == "taps":        # short convolutions: most weight on the newest tap, so signals pass
         taps = noise * 0.2
         taps[..., -1] += 1.0

@@ -416,7 +416,8 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
 
 
 def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, q_heads, kv_heads,
-                     head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None, num_decode=None, max_ctx=None):
+                     head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None, num_decode=None, max_ctx=None,
+                     softcap=None, head_gate=False):
     block_size = key_pages.shape[2]
     groups = q_heads // kv_heads
     for s in range(num_seqs):
@@ -437,13 +438,17 @@ def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table,
                 g = h // groups
                 qv = q[a + i, h * head_dim:(h + 1) * head_dim].float()
                 scores = (keys[g, first:p + 1] @ qv) * scale
+                if softcap is not None:
+                    scores = softcap * torch.tanh(scores / softcap)
                 top = scores.max()
                 if sink is not None:
                     top = torch.maximum(top, sink[h])
                 e = torch.exp(scores - top)
                 denom = e.sum() + (torch.exp(sink[h] - top) if sink is not None else 0.0)
                 o = (e / denom) @ values[g, first:p + 1]
-                if gate is not None:
+                if gate is not None and head_gate:
+                    o = o * torch.sigmoid(gate[a + i, h].float())
+                elif gate is not None:
                     o = o * torch.sigmoid(gate[a + i, h * value_dim:(h + 1) * value_dim].float())
                 out[a + i, h * value_dim:(h + 1) * value_dim] = o.to(out.dtype)
     return out
@@ -504,6 +509,113 @@ def mlstm_gate_scan(gates, bias, cap, maximum, cu_q, state_slots, out, *, num_se
     return out
 
 
+def hyper_norm(streams, update, mix, share, read, weight, bias, eps, out, rows=None, store=True, rms=False):
+    count = streams.shape[0]
+    x = streams
+    if update is not None:
+        y = _sum_parts(update)
+        m = torch.eye(count) if mix is None else mix
+        sh = torch.ones(count) if share is None else share
+        x = torch.einsum("sr,stw->rtw", m, streams) + sh[:, None, None] * y[None]
+        if store and rows is None:
+            streams.copy_(x)
+    if out is None:
+        return None
+    u = x.sum(0) if read is None else torch.einsum("s,stw->tw", read, x)
+    if rows is not None:
+        u = u[rows.long()]
+    if rms:
+        z = u * torch.rsqrt(u.square().mean(-1, keepdim=True) + eps) * weight
+    else:
+        centred = u - u.mean(-1, keepdim=True)
+        z = centred * torch.rsqrt(centred.square().mean(-1, keepdim=True) + eps) * weight
+    if bias is not None:
+        z = z + bias
+    out.copy_(z.to(out.dtype))
+    return out
+
+
+def embed_token_pairs(ids, table, pair_table, positions, token_seq, cu_q, state_slots, previous, out, *, num_seqs, buckets,
+                      mul_prev, mul_cur):
+    for t in range(ids.numel()):
+        cur = int(ids[t])
+        if int(positions[t]) == 0:
+            row = buckets
+        else:
+            s = int(token_seq[t])
+            prev = int(ids[t - 1]) if t > int(cu_q[s]) else int(previous[int(state_slots[s]), 0])
+            row = (prev * mul_prev + cur * mul_cur) % buckets
+        out[t] = table[cur].float() + pair_table[row].float()
+    for s in range(num_seqs):
+        if int(cu_q[s + 1]) > int(cu_q[s]):
+            previous[int(state_slots[s]), 0] = ids[int(cu_q[s + 1]) - 1]
+    return out
+
+
+def scale_rows(x, factor):
+    return x.mul_(factor)
+
+
+def whole_norm_rope_write(qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, key_pages, value_pages, q_out, *,
+                          q_heads, kv_heads, head_dim, value_dim, rotary_dim, eps, magnitude=1.0, write_kv=True):
+    tokens = qkv.shape[0]
+    q_size, k_size, v_size = q_heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
+
+    def prepare(x, weight, heads):
+        x = x.float()
+        x = (x * torch.rsqrt(x.square().mean(-1, keepdim=True) + eps) * weight).view(tokens, heads, head_dim)
+        if rotary_dim:
+            half = rotary_dim // 2
+            angle = positions.float().view(-1, 1, 1) * inv_freq.view(1, 1, half)
+            cos, sin = angle.cos() * magnitude, angle.sin() * magnitude
+            lo, hi = x[..., :half], x[..., half:rotary_dim]
+            x = torch.cat((lo * cos - hi * sin, hi * cos + lo * sin, x[..., rotary_dim:]), dim=-1)
+        return x
+
+    q_out.copy_(prepare(qkv[:, :q_size], q_weight, q_heads).reshape(tokens, q_size).to(q_out.dtype))
+    if not write_kv:
+        return
+    k = prepare(qkv[:, q_size:q_size + k_size], k_weight, kv_heads).to(qkv.dtype)
+    v = qkv[:, q_size + k_size:q_size + k_size + v_size].view(tokens, kv_heads, value_dim)
+    block_size = key_pages.shape[2]
+    for t in range(tokens):
+        pos = int(positions[t])
+        page = int(block_table[int(token_seq[t]), pos // block_size])
+        assert page >= 0, "token without a page"
+        key_pages[page, :, pos % block_size] = k[t]
+        value_pages[page, :, :, pos % block_size] = v[t]
+
+
+def moe_route(x, router_weight, router_bias, top):
+    z = x.float() @ router_weight.float().T
+    if router_bias is not None:
+        z = z + router_bias
+    best = torch.topk(z, top, dim=-1)
+    return best.indices.to(torch.int32), torch.softmax(best.values, dim=-1)
+
+
+def _gated(g, u, limit, alpha):
+    g = g.clamp(max=limit)
+    return g * torch.sigmoid(alpha * g) * (u.clamp(-limit, limit) + 1.0)
+
+
+def moe_experts(x, chosen, weights, gate_up, down, out, *, limit, alpha):
+    inner = gate_up.shape[1] // 2
+    for t in range(x.shape[0]):
+        for k in range(chosen.shape[1]):
+            e = int(chosen[t, k])
+            gu = gate_up[e].float() @ x[t].float()
+            act = _gated(gu[:inner], gu[inner:], limit, alpha).to(x.dtype).float()
+            out[k, t] = weights[t, k] * (down[e].float() @ act)
+    return out
+
+
+def linear_gated(x, gate_up_weight, *, limit, alpha):
+    gu = linear(x, gate_up_weight).float()
+    inner = gu.shape[1] // 2
+    return _gated(gu[:, :inner], gu[:, inner:], limit, alpha).to(x.dtype)
+
+
 def decode_prepare_supported(*args, **kwargs):
     return False        # on the CPU a step of single tokens takes the two references below in turn
 
@@ -520,7 +632,8 @@ DECODE_SPLITS_TESTED = tuple(range(1, 65))
 NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
          "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_filtered_rows",
          "cast_rows", "add_bias", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
-         "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan")
+         "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan",
+         "hyper_norm", "embed_token_pairs", "scale_rows", "whole_norm_rope_write", "moe_route", "moe_experts", "linear_gated")
 
 
 def install(monkeypatch):
