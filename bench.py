@@ -112,6 +112,8 @@ def parse_args():
     parser.add_argument("--points", default=None, help="other decode batch sizes to report")
     parser.add_argument("--widths", default="1024,2048,4096",
                         help="--phase design: model widths at which Mazanex and Qwen3 are measured side by side")
+    parser.add_argument("--design", choices=("mazanex", "rekezen"), default="mazanex",
+                        help="--phase design: which design is measured beside Qwen3")
     parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro", "check", "design"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
     parser.add_argument("--through", choices=("step", "scheduler"), default="step",
@@ -306,8 +308,31 @@ def design_configs(width: int, layers: int) -> dict:
     return {"Mazanex": mazanex, "Qwen3": qwen3}
 
 
+def rekezen_configs(width: int, layers: int) -> dict:
+    """Rekezen and Qwen3 at one width: heads of 128 in groups of four, the same vocabulary and layer
+    count.  Rekezen's feed-forward is a mixture of eight experts as wide as the model, of which a token
+    takes two, beside a shared one of the same size: three widths of active feed-forward a token, as
+    many as Qwen3's dense one.  Every second layer reads the keys and values of the layer before it;
+    four residual streams; a table of token pairs beside the embedding."""
+    heads = max(4, width // 128)
+
+    def mixer(index):
+        sizes = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+                 "rot": {"dims": 64, "base": 100000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+        if index % 2:
+            sizes["kv_from"] = index - 1
+        return sizes
+
+    mlp = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": width, "limit": 7.0},
+           "shared": {"ff": width, "limit": 7.0}}
+    rekezen = {"architecture": "Rekezen", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "streams": 4,
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 36313, "mul_cur": 27191}}, "logit_scale": 1.0,
+               "layers": [{"type": "attention", "mixer": mixer(i), "mlp": mlp} for i in range(layers)]}
+    return {"Rekezen": rekezen, "Qwen3": design_configs(width, layers)["Qwen3"]}
+
+
 def design_comparison(args) -> int:
-    """Prefill and decode throughput of Mazanex beside Qwen3 (the closest existing model) at equal
+    """Prefill and decode throughput of Mazanex (or, with ``--design rekezen``, Rekezen) beside Qwen3 (the closest existing model) at equal
     width, layer count, feed-forward size and vocabulary; random weights, one JSON line a model and width."""
     import torch
 
@@ -321,7 +346,7 @@ def design_comparison(args) -> int:
     prompt_len = args.prompt_len or 1024
     generator = torch.Generator().manual_seed(args.seed)
     for width in (int(w) for w in args.widths.split(",")):
-        for label, raw in design_configs(width, layers).items():
+        for label, raw in (rekezen_configs if args.design == "rekezen" else design_configs)(width, layers).items():
             config = load_model_config(raw)
             model = random_model(config, args.seed, dtype=dtype, device=device)
             pages = -(-(max(args.prefill_tokens, prompt_len) + args.steps + args.warmup + 16) // args.block_size)

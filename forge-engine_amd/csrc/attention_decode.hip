@@ -100,14 +100,14 @@ struct Prepare {
 
 // MODE 0: finished queries; 1: PREPARE from the projection's bfloat16 output; 2: PREPARE from its
 // float32 partial sums.
-template <int D, int MODE>
+template <int D, int MODE, bool CAP = false>
 __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* key_pages,
     const bf16_t* value_pages, bf16_t* __restrict__ out, long long out_stride,
     float* part_o, float* part_ml, int* __restrict__ counters, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
     int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2,
-    Prepare prep, int chunk, const float* __restrict__ sink) {
+    Prepare prep, int chunk, const float* __restrict__ sink, float cap_ratio) {
   constexpr bool PREPARE = MODE != 0, FROM_SUMS = MODE == 2;
   const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
@@ -258,7 +258,12 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int key = b * KEYS + 8 * lq + j;
-      const float v = st[j >> 2][j & 3] * scale_log2;
+      float raw = st[j >> 2][j & 3];
+      // a soft cap: the score after the scale becomes cap * tanh(score / cap); cap_ratio = cap / scale, and
+      // tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1)
+      if constexpr (CAP)
+        raw = cap_ratio * (1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(raw * (2.f * 1.4426950408889634f / cap_ratio)) + 1.f));
+      const float v = raw * scale_log2;
       s[j] = (key >= k_begin && key < cached) ? v : -INFINITY;
       mx = fmaxf(mx, s[j]);
     }
@@ -573,8 +578,9 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
                          const int* cu_q, const int* ctx_len, const int* block_table, int table_stride,
                          int num_seqs, int kv_heads, int groups, int head_dim, int block_size,
                          int num_blocks, int window, float scale, int splits, const Prepare* prep,
-                         int chunk, const float* sink, hipStream_t stream) {
+                         int chunk, const float* sink, hipStream_t stream, float softcap = 0.f) {
   if (num_seqs <= 0) return FE_OK;
+  if (softcap < 0.f || (softcap > 0.f && (prep || !(scale > 0.f)))) return FE_BAD_ARGUMENT;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
   if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
   if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
@@ -591,8 +597,16 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
 #define FE_GO(DD, MODE)                                                                                    \
   paged_decode_kernel<DD, MODE><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none, chunk, sink)
-  if (prep && prep->num_sums > 0) {
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none, chunk, sink, 0.f)
+#define FE_GO_CAPPED(DD)                                                                                   \
+  paged_decode_kernel<DD, 0, true><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, none, chunk, sink, softcap / scale)
+  if (softcap > 0.f) {
+    if (head_dim == 64) FE_GO_CAPPED(64);
+    else if (head_dim == 128) FE_GO_CAPPED(128);
+    else FE_GO_CAPPED(256);
+  } else if (prep && prep->num_sums > 0) {
     if (head_dim == 64) FE_GO(64, 2);
     else if (head_dim == 128) FE_GO(128, 2);
     else FE_GO(256, 2);
@@ -606,6 +620,7 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
     else FE_GO(256, 0);
   }
 #undef FE_GO
+#undef FE_GO_CAPPED
   return fe_check_launch();
 }
 
@@ -641,6 +656,21 @@ extern "C" int fe_paged_attention_decode_masked(const void* q, long long q_strid
   return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
                        ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
                        num_blocks, window, scale, splits, nullptr, chunk, sink, stream);
+}
+
+// The same with a soft cap on the scores: after the scale they become softcap * tanh(score / softcap).
+extern "C" int fe_paged_attention_decode_capped(const void* q, long long q_stride, const void* key_pages,
+                                                const void* value_pages, void* out, long long out_stride,
+                                                float* part_o, float* part_ml, int* counters, const int* cu_q,
+                                                const int* ctx_len, const int* block_table, int table_stride,
+                                                int num_seqs, int kv_heads, int groups, int head_dim,
+                                                int block_size, int num_blocks, int window, int chunk,
+                                                const float* sink, float scale, float softcap, int splits,
+                                                hipStream_t stream) {
+  if (!(softcap > 0.f)) return FE_BAD_ARGUMENT;
+  return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
+                       ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
+                       num_blocks, window, scale, splits, nullptr, chunk, sink, stream, softcap);
 }
 
 // The same for a batch in which EVERY sequence brings one token, straight from the fused

@@ -133,13 +133,13 @@ __device__ __forceinline__ int wave_most(int v) {
   return __builtin_amdgcn_readfirstlane(max((int)r[0], (int)r[1]));
 }
 
-template <int D, int KG, int RM>
+template <int D, int KG, int RM, bool CAP = false>
 __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_kernel(   // RM = 1: four waves a SIMD (128 registers), RM = 2: two
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
-    float scale_log2, int num_seqs, int heads_per_xcd, int chunk, const float* __restrict__ sink) {
+    float scale_log2, int num_seqs, int heads_per_xcd, int chunk, const float* __restrict__ sink, float cap_ratio) {
   const int block_mask = (1 << block_shift) - 1;
   constexpr int BM = 64 * RM;
   constexpr int KC = D / 32;            // MFMA k-steps over the head dim (scores)
@@ -365,7 +365,21 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
       if (half == 0) { pw[rm][blk].x = lo; pw[rm][blk].y = hi; } else { pw[rm][blk].z = lo; pw[rm][blk].w = hi; }
     }
   };
+  // CAP: scores, after the scale, are bounded as cap * tanh(score / cap).  With cap_ratio = cap / scale the raw
+  // score s becomes cap_ratio * tanh(s / cap_ratio), which the scale then takes to the bounded score; tanh(x) =
+  // 1 - 2 / (2^(2 x log2 e) + 1), before the masks put their infinities in.
+  auto cap_scores = [&](floatx4 (&st)[RM][2][2]) {
+    const float to_exponent = 2.f * 1.4426950408889634f / cap_ratio;
+#pragma unroll
+    for (int rm = 0; rm < RM; ++rm)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const float v = st[rm][j >> 3][(j >> 2) & 1][j & 3];
+        st[rm][j >> 3][(j >> 2) & 1][j & 3] = cap_ratio * (1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(v * to_exponent) + 1.f));
+      }
+  };
   auto softmax = [&](int key_base, floatx4 (&st)[RM][2][2], uintx4 (&pw)[RM][2]) {
+    if constexpr (CAP) cap_scores(st);
     if (is_edge(key_base)) mask_edges(key_base, st);
 #pragma unroll
     for (int rm = 0; rm < RM; ++rm)
@@ -635,6 +649,11 @@ extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stri
                                                  int groups, int head_dim, int block_size, int num_blocks,
                                                  int window, int chunk, const float* sink, float scale, int key_groups,
                                                  int row_sets, int total_q, hipStream_t stream);
+static int launch_prefill(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
+                          long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
+                          int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
+                          int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
+                          float softcap, int key_groups, int row_sets, int total_q, hipStream_t stream);
 
 extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, const void* key_pages,
                                                  const void* value_pages, void* out, long long out_stride,
@@ -659,6 +678,30 @@ extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stri
                                                  int groups, int head_dim, int block_size, int num_blocks,
                                                  int window, int chunk, const float* sink, float scale, int key_groups,
                                                  int row_sets, int total_q, hipStream_t stream) {
+  return launch_prefill(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len, block_table, table_stride,
+                        num_seqs, max_q_len, kv_heads, groups, head_dim, block_size, num_blocks, window, chunk, sink,
+                        scale, 0.f, key_groups, row_sets, total_q, stream);
+}
+
+// The same with a soft cap on the scores: after the scale they become softcap * tanh(score / softcap).
+extern "C" int fe_paged_attention_prefill_capped(const void* q, long long q_stride, const void* key_pages,
+                                                 const void* value_pages, void* out, long long out_stride,
+                                                 const int* cu_q, const int* ctx_len, const int* block_table,
+                                                 int table_stride, int num_seqs, int max_q_len, int kv_heads,
+                                                 int groups, int head_dim, int block_size, int num_blocks,
+                                                 int window, int chunk, const float* sink, float scale, float softcap,
+                                                 int key_groups, int row_sets, int total_q, hipStream_t stream) {
+  if (!(softcap > 0.f) || !(scale > 0.f)) return FE_BAD_ARGUMENT;
+  return launch_prefill(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len, block_table, table_stride,
+                        num_seqs, max_q_len, kv_heads, groups, head_dim, block_size, num_blocks, window, chunk, sink,
+                        scale, softcap, key_groups, row_sets, total_q, stream);
+}
+
+static int launch_prefill(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
+                          long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
+                          int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
+                          int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
+                          float softcap, int key_groups, int row_sets, int total_q, hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
   if (chunk < 0) return FE_BAD_ARGUMENT;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
@@ -693,10 +736,16 @@ extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stri
   // 4,096 cached ones 72 -> 53 us, one prompt of 512 tokens 13.5 -> 12.5 us) and the portions span at
   // least two tiles.
   if (key_groups == 0) key_groups = (row_sets == 1 && (long long)heads * filled_of(64) <= KEY_GROUPS_MAX_BLOCKS && max_q_len >= 128) ? 2 : 1;
-#define FE_GO(DD, GG, RR)                                                                                            \
-  paged_prefill_kernel<DD, GG, RR><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+  const float cap_ratio = softcap > 0.f ? softcap / scale : 0.f;
+#define FE_GO_C(DD, GG, RR, CC)                                                                                      \
+  paged_prefill_kernel<DD, GG, RR, CC><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
-      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink)
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink, cap_ratio)
+#define FE_GO(DD, GG, RR)                          \
+  do {                                             \
+    if (softcap > 0.f) FE_GO_C(DD, GG, RR, true);  \
+    else FE_GO_C(DD, GG, RR, false);               \
+  } while (0)
 #define FE_GO_D(DD)                                          \
   if (key_groups == 1 && row_sets == 1) FE_GO(DD, 1, 1);      \
   else if (row_sets == 1) FE_GO(DD, 2, 1);                    \
@@ -705,5 +754,6 @@ extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stri
   if (head_dim == 64) { FE_GO_D(64); } else { FE_GO_D(128); }
 #undef FE_GO_D
 #undef FE_GO
+#undef FE_GO_C
   return fe_check_launch();
 }

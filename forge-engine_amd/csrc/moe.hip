@@ -118,15 +118,16 @@ __device__ __forceinline__ float gated(float g, float u, float limit, float alph
 }
 
 // The expert and the first sorted row of this block's row tile; false if the slot is beyond the tiles.
+template <int ROWS = BM>
 __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E, int slot, int& expert, int& row0,
                                           int& row_end) {
   int tiles = 0;
   for (int e = 0; e < E; ++e) {
     const int begin = offsets[e], end = offsets[e + 1];
-    const int mine = (end - begin + BM - 1) / BM;
+    const int mine = (end - begin + ROWS - 1) / ROWS;
     if (slot < tiles + mine) {
       expert = e;
-      row0 = begin + (slot - tiles) * BM;
+      row0 = begin + (slot - tiles) * ROWS;
       row_end = end;
       return true;
     }
@@ -217,6 +218,91 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   }
 }
 
+// The same two products on the matrix cores, for bfloat16 with K a multiple of 32: a block takes 64 sorted
+// rows of one expert and 64 output columns (MODE 0: 64 gate columns and their 64 up columns), K in steps
+// of 32.  The rows go through LDS (two stages, one barrier a step; rows 80 bytes apart so that the
+// 16-byte reads of a fragment spread over the banks), the weight goes straight from memory into the
+// MFMA operand: wave w owns columns 16 w .. 16 w + 15 and all four 16-row tiles.  Both operands of the
+// next step are requested before this step's products.  A result lane holds rows 4 (lane / 16) + i of a
+// tile at column lane % 16.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
+#define TM 64
+#define TN 64
+#define TK 32
+#define TPAD 40
+
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
+    const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
+    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][TM][TPAD];
+  __shared__ int pair_of[TM];
+  int expert, row0, row_end;
+  if (!find_tile<TM>(offsets, E, blockIdx.x, expert, row0, row_end)) return;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 16, lq = lane / 16;
+  const int n0 = blockIdx.y * TN;
+  if (tid < TM) pair_of[tid] = row0 + tid < row_end ? order[row0 + tid] : -1;
+  __syncthreads();
+  // this thread's 16 bytes of a step's rows: row tid / 4, k chunk tid % 4
+  const int my_row = tid / 4, my_chunk = tid % 4;
+  const int my_pair = pair_of[my_row];
+  const size_t src = my_pair < 0 ? 0 : (MODE == 0 ? (size_t)(my_pair / top) : (size_t)(row0 + my_row));
+  const bf16_t* a_at = a + src * K + my_chunk * 8;
+  const int n = n0 + wave * 16 + lr;
+  const size_t w_rows = MODE == 0 ? 2 * (size_t)N : (size_t)N;
+  const bf16_t* wg_at = w + ((size_t)expert * w_rows + min(n, N - 1)) * K + lq * 8;
+  const bf16_t* wu_at = wg_at + (MODE == 0 ? (size_t)N * K : 0);
+  floatx4 acc_g[4], acc_u[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) acc_g[mt] = acc_u[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const uintx4 zero = {0u, 0u, 0u, 0u};
+  uintx4 a_reg = *(const uintx4*)a_at;
+  uintx4 wg_reg = *(const uintx4*)wg_at, wu_reg = *(const uintx4*)wu_at;
+  *(uintx4*)&As[0][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_reg;
+  __syncthreads();
+  const int steps = K / TK;
+  for (int step = 0; step < steps; ++step) {
+    const int stage = step & 1;
+    const int next = min(step + 1, steps - 1) * TK;      // the last step fetches its own operands again: no branch around a load
+    const uintx4 a_next = *(const uintx4*)(a_at + next);
+    const uintx4 wg_next = *(const uintx4*)(wg_at + next);
+    const uintx4 wu_next = *(const uintx4*)(wu_at + next);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const bf16x8 rows = *(const bf16x8*)&As[stage][mt * 16 + lr][lq * 8];
+      acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wg_reg), acc_g[mt], 0, 0, 0);
+      if (MODE == 0)
+        acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wu_reg), acc_u[mt], 0, 0, 0);
+    }
+    *(uintx4*)&As[stage ^ 1][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_next;
+    wg_reg = wg_next;
+    wu_reg = wu_next;
+    __syncthreads();
+  }
+  if (n >= N) return;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = mt * 16 + lq * 4 + i;
+      const int pair = pair_of[r];
+      if (pair < 0) continue;
+      if (MODE == 0) {
+        act[(size_t)(row0 + r) * N + n] = float_to_bf16(gated(acc_g[mt][i], acc_u[mt][i], limit, alpha));
+      } else {
+        const int token = pair / top, choice = pair - token * top;
+        out[((size_t)choice * tokens + token) * N + n] = acc_g[mt][i] * pair_weight[pair];
+      }
+    }
+}
+
+static bool mfma_fits(const void* a, const void* w, int K) {
+  return K % TK == 0 && ((((uintptr_t)a) | ((uintptr_t)w)) & 15) == 0;
+}
+
 extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, const int* offsets, const int* order, void* act,
                               int tokens, int top, int experts, int hidden, int inner, float limit, float alpha,
                               hipStream_t stream) {
@@ -227,6 +313,10 @@ extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, con
   if (dtype == FE_F32)
     moe_grouped_kernel<float, 0><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, offsets, order, nullptr,
                                                            (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha);
+  else if (dtype == FE_BF16 && mfma_fits(x, gate_up, hidden))
+    moe_grouped_mfma_kernel<0><<<dim3((unsigned)(pairs / TM + experts), (unsigned)((inner + TN - 1) / TN)), 256, 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr, (bf16_t*)act, nullptr, experts, inner, hidden, top,
+        tokens, limit, alpha);
   else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr,
                                                             (bf16_t*)act, nullptr, experts, inner, hidden, top, tokens, limit,
@@ -246,6 +336,10 @@ extern "C" int fe_moe_down(const void* act, const void* down, int dtype, const i
   if (dtype == FE_F32)
     moe_grouped_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, offsets, order, pair_weight,
                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f);
+  else if (dtype == FE_BF16 && mfma_fits(act, down, inner))
+    moe_grouped_mfma_kernel<1><<<dim3((unsigned)(pairs / TM + experts), (unsigned)((hidden + TN - 1) / TN)), 256, 0, stream>>>(
+        (const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight, nullptr, out, experts, hidden, inner, top, tokens,
+        0.f, 0.f);
   else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight,
                                                             nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f);

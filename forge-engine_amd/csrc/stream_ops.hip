@@ -244,26 +244,27 @@ extern "C" int fe_add_bias(float* update, const float* bias, int rows, int width
 }
 
 // ---------------------------------------------------------------- output gate
-// out[t][c] *= sigmoid(gate[t][c]), gate rows `gate_stride` elements apart
+// out[t][c] *= sigmoid(gate[t][c / share]), gate rows `gate_stride` elements apart; `share` consecutive
+// outputs take one gate (1: a gate per element; a head's width: a gate per head)
 template <typename T>
 __global__ void sigmoid_gate_kernel(T* __restrict__ out, const T* __restrict__ gate, size_t gate_stride, int width,
-                                    long long count) {
+                                    long long count, int share) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count) return;
   const long long t = i / width;
   const int c = (int)(i - t * width);
-  const float g = load_as_float(gate + (size_t)t * gate_stride + c);
+  const float g = load_as_float(gate + (size_t)t * gate_stride + c / share);
   store_from_float(out + i, load_as_float(out + i) / (1.f + expf(-g)));
 }
 
 extern "C" int fe_sigmoid_gate(void* out, const void* gate, long long gate_stride, int dtype, int rows, int width,
-                               hipStream_t stream) {
+                               int share, hipStream_t stream) {
   if (rows <= 0) return FE_OK;
-  if (width <= 0 || gate_stride < width) return FE_BAD_ARGUMENT;
+  if (width <= 0 || share < 1 || width % share || gate_stride < width / share) return FE_BAD_ARGUMENT;
   const long long count = (long long)rows * width;
   const int blocks = (int)((count + 255) / 256);
-  if (dtype == FE_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gate, (size_t)gate_stride, width, count);
-  else if (dtype == FE_BF16) sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gate, (size_t)gate_stride, width, count);
+  if (dtype == FE_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gate, (size_t)gate_stride, width, count, share);
+  else if (dtype == FE_BF16) sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gate, (size_t)gate_stride, width, count, share);
   else return FE_BAD_ARGUMENT;
   return fe_check_launch();
 }

@@ -714,11 +714,12 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
                     window: int | None = None, num_decode: int | None = None,
                     max_ctx: int | None = None, splits: int | None = None, chunk: int | None = None,
-                    sink: Tensor | None = None) -> Tensor:
+                    sink: Tensor | None = None, softcap: float | None = None) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
 
-    ``chunk`` (a token reads keys of its own run of that many positions only) and ``sink``
-    (float32 [Hq]: exp(sink_h) joins head h's softmax denominator) are served by the two
+    ``chunk`` (a token reads keys of its own run of that many positions only), ``sink``
+    (float32 [Hq]: exp(sink_h) joins head h's softmax denominator) and ``softcap`` (scores, after
+    the scale, become cap * tanh(score / cap)) are served by the two
     matrix-core kernels alone: a call that brings either for sizes those do not take is refused
     (``masked_attention`` routes such sizes to the vector-ALU kernel that knows both).
 
@@ -764,10 +765,12 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                   and q.data_ptr() % 16 == 0 and q_stride % 8 == 0)      # the fast kernels read 16 bytes at a time
     fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
     fast_prefill = bf16_pages and head_dim in (64, 128)
-    masked = chunk is not None or sink is not None
+    masked = chunk is not None or sink is not None or softcap is not None
     if masked:
         if (any_single and not fast_decode) or (any_longer and not fast_prefill):
-            raise KernelError("chunks and sinks are served by the matrix-core attention kernels only")
+            raise KernelError("chunks, sinks and soft caps are served by the matrix-core attention kernels only")
+        if softcap is not None and not (softcap > 0.0 and scale > 0.0):
+            raise KernelError("softcap and scale must be positive")
         if sink is not None:
             _gpu(sink, "sink", torch.float32)
             if sink.shape != (q_heads,):
@@ -799,20 +802,22 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
             part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=q.device)
             counters = _split_counters(q.device, num_seqs * kv_heads)
         mask = (c_int(chunk or 0), _ptr(sink)) if masked else ()
-        _call("attention_decode", "fe_paged_attention_decode_masked" if masked else "fe_paged_attention_decode",
-              _ptr(q), c_longlong(q_stride),
+        cap = (c_float(softcap),) if softcap is not None else ()
+        name = "fe_paged_attention_decode_capped" if cap else "fe_paged_attention_decode_masked" if masked else "fe_paged_attention_decode"
+        _call("attention_decode", name, _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(part_o),
               _ptr(part_ml), _ptr(counters), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
               c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), c_int(splits), _stream())
+              c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), *cap, c_int(splits), _stream())
     if any_longer and fast_prefill:
         mask = (c_int(chunk or 0), _ptr(sink)) if masked else ()
-        _call("attention_prefill", "fe_paged_attention_prefill_masked" if masked else "fe_paged_attention_prefill",
-              _ptr(q), c_longlong(q_stride),
+        cap = (c_float(softcap),) if softcap is not None else ()
+        name = "fe_paged_attention_prefill_capped" if cap else "fe_paged_attention_prefill_masked" if masked else "fe_paged_attention_prefill"
+        _call("attention_prefill", name, _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), c_int(PREFILL_KEY_GROUPS), c_int(PREFILL_ROW_SETS),
+              c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), *cap, c_int(PREFILL_KEY_GROUPS), c_int(PREFILL_ROW_SETS),
               c_int(tokens), _stream())
     # whatever the two fast kernels did not take: single tokens go to the vector-ALU decode kernel where
     # it can read four elements at a time, the rest to the general kernel
@@ -1288,15 +1293,14 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
         raise KernelError("softcap must be positive")
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
-    if (softcap is None and not head_gate
-            and q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
+    if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
             and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
         paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
                         q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
-                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink)
+                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink, softcap=softcap)
         if gate is not None:
             _call("stream_ops", "fe_sigmoid_gate", _ptr(out), _ptr(gate), c_longlong(gate_stride), c_int(_code(out.dtype)),
-                  c_int(tokens), c_int(q_heads * value_dim), _stream())
+                  c_int(tokens), c_int(q_heads * value_dim), c_int(value_dim if head_gate else 1), _stream())
         return out
     _call("attention_masked", "fe_masked_attention", _ptr(q), c_int(_code(q.dtype)), c_longlong(q_stride), _ptr(key_pages),
           _ptr(value_pages), _ptr(out), _ptr(gate), c_longlong(gate_stride), _ptr(sink), _ptr(cu_q), _ptr(ctx_len),
