@@ -1,12 +1,13 @@
 // A mixture of experts on the device: routing, the sort of (token, choice) pairs by expert, and
 // two grouped matrix products over the sorted rows.  Nothing is decided on the host.
 //
-//   fe_moe_route:    z = W_r x + b (float32), the `top` largest per token, softmax over those alone
+//   fe_moe_select:   from router logits (float32): bias added, the `top` largest per token, softmax over those alone
 //   fe_moe_plan:     counts per expert, their prefix sums, and the pairs ordered by expert
 //   fe_moe_gate_up:  for every pair, act = min(g, L) * sigmoid(alpha min(g, L)) * (clamp(u, -L, L) + 1) with
 //                    g = W_gate[e] x, u = W_up[e] x of the pair's token and expert
 //   fe_moe_down:     out[choice][token] = weight * W_down[e] act   (float32; one part per choice, so
-//                    that the reader adds a token's experts up in a fixed order)
+//                    that the reader adds a token's experts up in a fixed order; the first choice's part
+//                    also takes what every token gets beside its experts, a shared expert's output)
 //   fe_gated_act:    the same activation over a dense [T, 2F] product (a shared expert)
 //
 // The grouped products tile the sorted rows 32 at a time within an expert (a tile never spans two
@@ -15,38 +16,30 @@
 // a block whose slot lies beyond the tiles there are returns at once.
 #include "common.h"
 
-#define ROUTE_WAVES 4
-
-template <typename T>
-__global__ __launch_bounds__(64 * ROUTE_WAVES) void moe_route_kernel(
-    const T* __restrict__ x, const T* __restrict__ router, const float* __restrict__ bias, int* __restrict__ chosen,
-    float* __restrict__ weights, int tokens, int H, int E, int top) {
-  extern __shared__ float logits[];     // [ROUTE_WAVES][E]
-  const int wave = threadIdx.x / FE_WAVE, lane = threadIdx.x % FE_WAVE;
-  const int t = blockIdx.x * ROUTE_WAVES + wave;
+// One thread per token over its row of router logits z [T, E] (float32, the product comes from the
+// caller): bias added, the `top` largest chosen one after the other (the largest first; among equals
+// the lowest index), weights = softmax over the chosen logits alone.
+__global__ void moe_select_kernel(const float* __restrict__ z, const float* __restrict__ bias, int* __restrict__ chosen,
+                                  float* __restrict__ weights, int tokens, int E, int top) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= tokens) return;
-  float* z = logits + wave * E;
-  const T* row = x + (size_t)t * H;
-  for (int e = 0; e < E; ++e) {
-    const T* w = router + (size_t)e * H;
-    float partial = 0.f;
-    for (int k = lane; k < H; k += FE_WAVE) partial = fmaf(load_as_float(row + k), load_as_float(w + k), partial);
-    const float total = wave_sum(partial);
-    if (lane == 0) z[e] = total + (bias ? bias[e] : 0.f);
-  }
-  if (lane != 0) return;
-  // the largest first; among equals the lowest index
+  const float* row = z + (size_t)t * E;
+  int picked[16];
   float best[16];
   float peak = 0.f, denom = 0.f;
   for (int k = 0; k < top; ++k) {
-    int arg = 0;
+    int arg = -1;
     float value = -INFINITY;
-    for (int e = 0; e < E; ++e)
-      if (z[e] > value) {
-        value = z[e];
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken = taken || picked[j] == e;
+      const float v = row[e] + (bias ? bias[e] : 0.f);
+      if (!taken && (arg < 0 || v > value)) {
+        value = v;
         arg = e;
       }
-    z[arg] = -INFINITY;
+    }
+    picked[k] = arg;
     chosen[(size_t)t * top + k] = arg;
     if (k == 0) peak = value;
     best[k] = expf(value - peak);
@@ -55,20 +48,11 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void moe_route_kernel(
   for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] = best[k] / denom;
 }
 
-extern "C" int fe_moe_route(const void* x, const void* router, int dtype, const float* bias, int* chosen, float* weights,
-                            int tokens, int hidden, int experts, int top, hipStream_t stream) {
+extern "C" int fe_moe_select(const float* logits, const float* bias, int* chosen, float* weights, int tokens, int experts,
+                             int top, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
-  if (hidden <= 0 || experts <= 0 || experts > 1024 || top < 1 || top > 16 || top > experts) return FE_BAD_ARGUMENT;
-  const int blocks = (tokens + ROUTE_WAVES - 1) / ROUTE_WAVES;
-  const size_t lds = (size_t)ROUTE_WAVES * experts * sizeof(float);
-  if (dtype == FE_F32)
-    moe_route_kernel<float><<<blocks, 64 * ROUTE_WAVES, lds, stream>>>((const float*)x, (const float*)router, bias, chosen,
-                                                                       weights, tokens, hidden, experts, top);
-  else if (dtype == FE_BF16)
-    moe_route_kernel<bf16_t><<<blocks, 64 * ROUTE_WAVES, lds, stream>>>((const bf16_t*)x, (const bf16_t*)router, bias, chosen,
-                                                                        weights, tokens, hidden, experts, top);
-  else
-    return FE_BAD_ARGUMENT;
+  if (experts <= 0 || experts > 1024 || top < 1 || top > 16 || top > experts) return FE_BAD_ARGUMENT;
+  moe_select_kernel<<<(tokens + 63) / 64, 64, 0, stream>>>(logits, bias, chosen, weights, tokens, experts, top);
   return fe_check_launch();
 }
 
@@ -117,6 +101,16 @@ __device__ __forceinline__ float gated(float g, float u, float limit, float alph
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
 }
 
+// A token's first choice also takes what every token gets beside its experts (a shared expert's output,
+// float32 [parts][tokens][N], added up in order first).
+__device__ __forceinline__ float with_extra(float v, int choice, const float* __restrict__ extra, int parts,
+                                            size_t part_stride, size_t at) {
+  if (choice != 0 || !extra) return v;
+  float sum = extra[at];
+  for (int p = 1; p < parts; ++p) sum += extra[p * part_stride + at];
+  return v + sum;
+}
+
 // The expert and the first sorted row of this block's row tile; false if the slot is beyond the tiles.
 template <int ROWS = BM>
 __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E, int slot, int& expert, int& row0,
@@ -143,7 +137,7 @@ template <typename T, int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const T* __restrict__ a, const T* __restrict__ w, const int* __restrict__ offsets, const int* __restrict__ order,
     const float* __restrict__ pair_weight, T* __restrict__ act, float* __restrict__ out, int E, int N, int K, int top,
-    int tokens, float limit, float alpha) {
+    int tokens, float limit, float alpha, const float* __restrict__ extra, int extra_parts) {
   __shared__ float As[BM][BK + 1];
   __shared__ float Ws[BN][BK + 1];
   __shared__ float Us[MODE == 0 ? BN : 1][BK + 1];
@@ -212,7 +206,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
         store_from_float(act + (size_t)(row0 + r) * N + n, gated(acc_g[i][j], acc_u[i][j], limit, alpha));
       } else {
         const int token = pair / top, choice = pair - token * top;
-        out[((size_t)choice * tokens + token) * N + n] = acc_g[i][j] * pair_weight[pair];
+        out[((size_t)choice * tokens + token) * N + n] =
+            with_extra(acc_g[i][j] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
       }
     }
   }
@@ -237,7 +232,8 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
     const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
-    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha) {
+    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
+    const float* __restrict__ extra, int extra_parts) {
   __shared__ __attribute__((aligned(16))) bf16_t As[2][TM][TPAD];
   __shared__ int pair_of[TM];
   int expert, row0, row_end;
@@ -259,29 +255,52 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) acc_g[mt] = acc_u[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const uintx4 zero = {0u, 0u, 0u, 0u};
-  uintx4 a_reg = *(const uintx4*)a_at;
-  uintx4 wg_reg = *(const uintx4*)wg_at, wu_reg = *(const uintx4*)wu_at;
-  *(uintx4*)&As[0][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_reg;
-  __syncthreads();
+  // Step s has its operands in register set s % DEPTH, requested DEPTH steps ahead (a step's arithmetic is far
+  // shorter than a trip to memory, and a launch of few blocks keeps the memory busy only through what each
+  // block has in flight).  The rows of step s + 1 go into the other LDS stage while step s multiplies; one
+  // barrier a step.  Whole rounds of DEPTH steps are straight-line code; steps beyond the last fetch the last
+  // step's operands again, so that no load stands under a branch.
+  constexpr int DEPTH = 4;
   const int steps = K / TK;
-  for (int step = 0; step < steps; ++step) {
-    const int stage = step & 1;
-    const int next = min(step + 1, steps - 1) * TK;      // the last step fetches its own operands again: no branch around a load
-    const uintx4 a_next = *(const uintx4*)(a_at + next);
-    const uintx4 wg_next = *(const uintx4*)(wg_at + next);
-    const uintx4 wu_next = *(const uintx4*)(wu_at + next);
+  uintx4 a_reg[DEPTH], wg_reg[DEPTH], wu_reg[DEPTH];
+  auto fetch = [&](int step, int set) {
+    const int at = min(step, steps - 1) * TK;
+    a_reg[set] = *(const uintx4*)(a_at + at);
+    wg_reg[set] = *(const uintx4*)(wg_at + at);
+    if (MODE == 0) wu_reg[set] = *(const uintx4*)(wu_at + at);
+  };
+  auto multiply = [&](int stage, int set) {
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       const bf16x8 rows = *(const bf16x8*)&As[stage][mt * 16 + lr][lq * 8];
-      acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wg_reg), acc_g[mt], 0, 0, 0);
+      acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wg_reg[set]), acc_g[mt], 0, 0, 0);
       if (MODE == 0)
-        acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wu_reg), acc_u[mt], 0, 0, 0);
+        acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wu_reg[set]), acc_u[mt], 0, 0, 0);
     }
-    *(uintx4*)&As[stage ^ 1][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_next;
-    wg_reg = wg_next;
-    wu_reg = wu_next;
-    __syncthreads();
+  };
+  auto stash = [&](int stage, int set) { *(uintx4*)&As[stage][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_reg[set]; };
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) fetch(u, u);
+  stash(0, 0);
+  __syncthreads();
+  int step = 0;
+  for (; step + DEPTH <= steps; step += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      multiply(u & 1, u);
+      stash((u + 1) & 1, (u + 1) % DEPTH);
+      fetch(step + u + DEPTH, u);
+      __syncthreads();
+    }
   }
+  const int left = steps - step;       // 0 .. DEPTH - 1, the same for every thread
+#pragma unroll
+  for (int u = 0; u < DEPTH - 1; ++u)
+    if (u < left) {
+      multiply(u & 1, u);
+      stash((u + 1) & 1, (u + 1) % DEPTH);
+      __syncthreads();
+    }
   if (n >= N) return;
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt)
@@ -294,7 +313,8 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
         act[(size_t)(row0 + r) * N + n] = float_to_bf16(gated(acc_g[mt][i], acc_u[mt][i], limit, alpha));
       } else {
         const int token = pair / top, choice = pair - token * top;
-        out[((size_t)choice * tokens + token) * N + n] = acc_g[mt][i] * pair_weight[pair];
+        out[((size_t)choice * tokens + token) * N + n] =
+            with_extra(acc_g[mt][i] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
       }
     }
 }
@@ -312,15 +332,15 @@ extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, con
   const dim3 grid((unsigned)(pairs / BM + experts), (unsigned)((inner + BN - 1) / BN));
   if (dtype == FE_F32)
     moe_grouped_kernel<float, 0><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, offsets, order, nullptr,
-                                                           (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha);
+                                                           (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha, nullptr, 0);
   else if (dtype == FE_BF16 && mfma_fits(x, gate_up, hidden))
     moe_grouped_mfma_kernel<0><<<dim3((unsigned)(pairs / TM + experts), (unsigned)((inner + TN - 1) / TN)), 256, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr, (bf16_t*)act, nullptr, experts, inner, hidden, top,
-        tokens, limit, alpha);
+        tokens, limit, alpha, nullptr, 0);
   else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr,
                                                             (bf16_t*)act, nullptr, experts, inner, hidden, top, tokens, limit,
-                                                            alpha);
+                                                            alpha, nullptr, 0);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();
@@ -328,21 +348,23 @@ extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, con
 
 extern "C" int fe_moe_down(const void* act, const void* down, int dtype, const int* offsets, const int* order,
                            const float* pair_weight, float* out, int tokens, int top, int experts, int hidden, int inner,
-                           hipStream_t stream) {
+                           const float* extra, int extra_parts, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
-  if (top < 1 || experts < 1 || experts > 1024 || hidden <= 0 || inner <= 0) return FE_BAD_ARGUMENT;
+  if (top < 1 || experts < 1 || experts > 1024 || hidden <= 0 || inner <= 0 || (extra && extra_parts < 1)) return FE_BAD_ARGUMENT;
   const long long pairs = (long long)tokens * top;
   const dim3 grid((unsigned)(pairs / BM + experts), (unsigned)((hidden + BN - 1) / BN));
   if (dtype == FE_F32)
     moe_grouped_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, offsets, order, pair_weight,
-                                                           nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f);
+                                                           nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, extra,
+                                                           extra_parts);
   else if (dtype == FE_BF16 && mfma_fits(act, down, inner))
     moe_grouped_mfma_kernel<1><<<dim3((unsigned)(pairs / TM + experts), (unsigned)((hidden + TN - 1) / TN)), 256, 0, stream>>>(
         (const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight, nullptr, out, experts, hidden, inner, top, tokens,
-        0.f, 0.f);
+        0.f, 0.f, extra, extra_parts);
   else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight,
-                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f);
+                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, extra,
+                                                           extra_parts);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();

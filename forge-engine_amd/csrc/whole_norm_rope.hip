@@ -1,5 +1,6 @@
 // From the projection's output to queries and cached keys and values, for attention that
-// normalises q and k over the whole projection: one block per token.
+// normalises q and k over the whole projection: one block per token, or, in a step of few tokens, one
+// per token and head.
 //   q <- q / sqrt(mean over all heads and dims of q^2 + eps) * w_q      (w_q as long as q; k likewise)
 //   the first R dims of every head turn by the token's position: dim i < R/2 pairs with i + R/2,
 //   (a, b) -> (a c - b s, b c + a s) with c = magnitude cos(p f_i), s = magnitude sin(p f_i)
@@ -55,23 +56,52 @@ __global__ __launch_bounds__(256) void whole_norm_rope_kernel(
     return v;
   };
 
-  T* qrow = q_out + (size_t)t * q_size;
-  for (int e = tid; e < q_size; e += 256) store_from_float(qrow + e, turned(row, q_weight, inv_q, e, e % D));
-  if (!write_kv) return;
-  const int seq = token_seq[t];
-  const int page = block_table[(size_t)seq * table_stride + pos / block_size];
-  if (page < 0 || page >= num_blocks) return;
-  const int slot = pos % block_size;
-  const T* krow = row + q_size;
-  for (int e = tid; e < kv_size; e += 256) {
-    const int h = e / D, d = e - h * D;
-    store_from_float(key_pages + (((size_t)page * kv_heads + h) * block_size + slot) * D + d,
-                     turned(krow, k_weight, inv_k, e, d));
+  // Units of work: the q heads, then the k heads, then the v heads.  A launch of many tokens gives a block
+  // all units of its token; one of few tokens spreads them over blockIdx.y (every block forms the sums of
+  // squares for itself), so that a step of a few single tokens still fills some of the chip.
+  const int units = q_heads + (write_kv ? 2 * kv_heads : 0);
+  int page = -1, slot = 0;
+  if (write_kv) {
+    const int seq = token_seq[t];
+    page = block_table[(size_t)seq * table_stride + pos / block_size];
+    if (page < 0 || page >= num_blocks) page = -1;
+    slot = pos % block_size;
   }
+  T* qrow = q_out + (size_t)t * q_size;
+  const T* krow = row + q_size;
   const T* vrow = krow + kv_size;
-  for (int e = tid; e < kv_heads * Dv; e += 256) {
-    const int h = e / Dv, d = e - h * Dv;
-    value_pages[(((size_t)page * kv_heads + h) * Dv + d) * block_size + slot] = vrow[e];
+  auto q_range = [&](int begin, int end) {
+    for (int e = begin + tid; e < end; e += 256) store_from_float(qrow + e, turned(row, q_weight, inv_q, e, e % D));
+  };
+  auto k_range = [&](int begin, int end) {
+    for (int e = begin + tid; e < end; e += 256) {
+      const int h = e / D, d = e - h * D;
+      store_from_float(key_pages + (((size_t)page * kv_heads + h) * block_size + slot) * D + d,
+                       turned(krow, k_weight, inv_k, e, d));
+    }
+  };
+  auto v_range = [&](int begin, int end) {
+    for (int e = begin + tid; e < end; e += 256) {
+      const int h = e / Dv, d = e - h * Dv;
+      value_pages[(((size_t)page * kv_heads + h) * Dv + d) * block_size + slot] = vrow[e];
+    }
+  };
+  if (gridDim.y == 1) {
+    q_range(0, q_size);
+    if (page >= 0) {
+      k_range(0, kv_size);
+      v_range(0, kv_heads * Dv);
+    }
+    return;
+  }
+  for (int unit = blockIdx.y; unit < units; unit += gridDim.y) {
+    if (unit < q_heads) {
+      q_range(unit * D, (unit + 1) * D);
+    } else if (page >= 0 && unit < q_heads + kv_heads) {
+      k_range((unit - q_heads) * D, (unit - q_heads + 1) * D);
+    } else if (page >= 0) {
+      v_range((unit - q_heads - kv_heads) * Dv, (unit - q_heads - kv_heads + 1) * Dv);
+    }
   }
 }
 
@@ -87,8 +117,10 @@ extern "C" int fe_whole_norm_rope_write(const void* qkv, int dtype, long long st
       rotary_dim > head_dim || rotary_dim > 256 || stride < need || !(eps > 0.f) || !q_weight || (rotary_dim && !inv_freq) ||
       (write_kv && (!k_weight || !key_pages || !value_pages || !block_table || block_size <= 0 || num_blocks <= 0)))
     return FE_BAD_ARGUMENT;
+  const int units = q_heads + (write_kv ? 2 * kv_heads : 0);
+  const dim3 grid(tokens, tokens <= 256 ? (units < 65535 ? units : 65535) : 1);
 #define LAUNCH(T)                                                                                                      \
-  whole_norm_rope_kernel<T><<<tokens, 256, 0, stream>>>((const T*)qkv, (size_t)stride, q_weight, k_weight, inv_freq,   \
+  whole_norm_rope_kernel<T><<<grid, 256, 0, stream>>>((const T*)qkv, (size_t)stride, q_weight, k_weight, inv_freq,   \
                                                         positions, token_seq, block_table, table_stride, (T*)key_pages, \
                                                         (T*)value_pages, (T*)q_out, q_heads, kv_heads, head_dim,       \
                                                         value_dim, rotary_dim, eps, magnitude, write_kv, block_size,   \

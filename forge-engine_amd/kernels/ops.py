@@ -1550,20 +1550,22 @@ def moe_route(x: Tensor, router_weight: Tensor, router_bias: Tensor | None, top:
         _gpu(router_bias, "router_bias", torch.float32)
         if router_bias.shape != (experts,):
             raise KernelError(f"router_bias must be [{experts}]")
+    logits = linear(x, router_weight, out_dtype=torch.float32)     # float32 accumulation, float32 logits
     chosen = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
-    _call("moe", "fe_moe_route", _ptr(x), _ptr(router_weight), c_int(_code(x.dtype)), _ptr(router_bias), _ptr(chosen),
-          _ptr(weights), c_int(tokens), c_int(hidden), c_int(experts), c_int(top), _stream())
+    _call("moe", "fe_moe_select", _ptr(logits), _ptr(router_bias), _ptr(chosen), _ptr(weights), c_int(tokens), c_int(experts),
+          c_int(top), _stream())
     return chosen, weights
 
 
 def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, down: Tensor, out: Tensor, *, limit: float,
-                alpha: float) -> Tensor:
+                alpha: float, extra: Tensor | None = None) -> Tensor:
     """out[k, t] = weights[t, k] * down[e] @ act, e = chosen[t, k], with ``act = min(g, limit) *
     sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)``, ``g = gate_up[e, :F] @ x[t]``,
     ``u = gate_up[e, F:] @ x[t]``.  x [T, H]; gate_up [E, 2F, H]; down [E, H, F]; out float32 [top, T, H]
-    (one part per choice).  The pairs are sorted by expert on the device and two grouped products run
-    over the sorted rows."""
+    (one part per choice).  ``extra`` (float32 [T, H] or [parts, T, H], added up in order): what every
+    token gets beside its experts; it joins the first choice's part.  The pairs are sorted by expert on the
+    device and two grouped products run over the sorted rows."""
     _gpu(x, "x")
     _gpu(chosen, "chosen", torch.int32)
     _gpu(weights, "weights", torch.float32)
@@ -1583,6 +1585,7 @@ def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, dow
         raise KernelError(f"out must be [{top}, {tokens}, {hidden}], got {tuple(out.shape)}")
     if not limit > 0.0:
         raise KernelError("limit must be positive")
+    extra_parts = 0 if extra is None else _parts_of(extra, tokens, hidden, "extra")
     pairs = tokens * top
     offsets = torch.empty(experts + 1, dtype=torch.int32, device=x.device)
     order = torch.empty(pairs, dtype=torch.int32, device=x.device)
@@ -1592,7 +1595,7 @@ def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, dow
     _call("moe", "fe_moe_gate_up", _ptr(x), _ptr(gate_up), code, _ptr(offsets), _ptr(order), _ptr(act), c_int(tokens), c_int(top),
           c_int(experts), c_int(hidden), c_int(inner), c_float(limit), c_float(alpha), _stream())
     _call("moe", "fe_moe_down", _ptr(act), _ptr(down), code, _ptr(offsets), _ptr(order), _ptr(weights), _ptr(out), c_int(tokens),
-          c_int(top), c_int(experts), c_int(hidden), c_int(inner), _stream())
+          c_int(top), c_int(experts), c_int(hidden), c_int(inner), _ptr(extra), c_int(extra_parts), _stream())
     return out
 
 

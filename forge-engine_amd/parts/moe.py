@@ -10,8 +10,8 @@ token takes.
 A step sorts its (token, choice) pairs by expert on the device and runs two grouped products over
 the sorted rows (gate and up with the activation as their ending, then down, weighted by the
 router); nothing is decided on the host, so steps are captured like any other.  The update comes
-back in parts, one per choice and the shared expert's behind them, which the next norm adds up in
-that order: a token's sum does not depend on what else is in the step.
+back in parts, one per choice (the shared expert's output joins the first), which the next norm adds
+up in that order: a token's sum does not depend on what else is in the step.
 """
 
 from __future__ import annotations
@@ -111,17 +111,13 @@ class RoutedExperts(FeedForward):
     def forward(self, x: Tensor, batch=None) -> Tensor:
         tokens = x.shape[0]
         chosen, weights = ops.moe_route(x, self.router_weight, self.router_bias, self.top)
-        parts = self.top + (1 if self.shared_size else 0)
-        update = torch.empty((parts, tokens, self.hidden_size), dtype=torch.float32, device=x.device)
-        ops.moe_experts(x, chosen, weights, self.gate_up, self.down, update[:self.top], limit=self.limit, alpha=self.alpha)
+        shared = None
         if self.shared_size:
             act = ops.linear_gated(x, self.shared_gate_up, limit=self.shared_limit, alpha=self.alpha)
             shared = ops.linear_update(act, self.shared_down)
-            if shared.dim() == 2:
-                update[self.top].copy_(shared)
-            else:           # the product came in parts of K itself
-                update = torch.cat([update[:self.top], shared])
-        return update
+        update = torch.empty((self.top, tokens, self.hidden_size), dtype=torch.float32, device=x.device)
+        return ops.moe_experts(x, chosen, weights, self.gate_up, self.down, update, limit=self.limit, alpha=self.alpha,
+                               extra=shared)
 
     def kernel_libraries(self):
         return {"moe", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}

@@ -599,7 +599,7 @@ def _gated(g, u, limit, alpha):
     return g * torch.sigmoid(alpha * g) * (u.clamp(-limit, limit) + 1.0)
 
 
-def moe_experts(x, chosen, weights, gate_up, down, out, *, limit, alpha):
+def moe_experts(x, chosen, weights, gate_up, down, out, *, limit, alpha, extra=None):
     inner = gate_up.shape[1] // 2
     for t in range(x.shape[0]):
         for k in range(chosen.shape[1]):
@@ -607,6 +607,8 @@ def moe_experts(x, chosen, weights, gate_up, down, out, *, limit, alpha):
             gu = gate_up[e].float() @ x[t].float()
             act = _gated(gu[:inner], gu[inner:], limit, alpha).to(x.dtype).float()
             out[k, t] = weights[t, k] * (down[e].float() @ act)
+    if extra is not None:
+        out[0] += _sum_parts(extra)
     return out
 
 

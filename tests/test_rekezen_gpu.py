@@ -160,6 +160,12 @@ def test_mixture_of_experts_kernels(tokens, hidden, experts, top, inner, dtype):
     got = ops.moe_experts(x.to(DEV), chosen, weights, gate_up.to(DEV), down.to(DEV), torch.empty(top, tokens, hidden, device=DEV),
                           limit=1.2, alpha=1.702)
     close(got, want, dtype)
+    for extra in (torch.randn(tokens, hidden, generator=g), torch.randn(3, tokens, hidden, generator=g)):   # what every token gets beside
+        want = refs.moe_experts(x, want_chosen, want_weights, gate_up, down, torch.empty(top, tokens, hidden), limit=1.2, alpha=1.702,
+                                extra=extra)
+        got = ops.moe_experts(x.to(DEV), chosen, weights, gate_up.to(DEV), down.to(DEV), torch.empty(top, tokens, hidden, device=DEV),
+                              limit=1.2, alpha=1.702, extra=extra.to(DEV))
+        close(got, want, dtype)
     shared = (torch.randn(2 * inner, hidden, generator=g) * 0.3).to(dtype)
     close(ops.linear_gated(x.to(DEV), shared.to(DEV), limit=0.8, alpha=1.702), refs.linear_gated(x, shared, limit=0.8, alpha=1.702), dtype)
 
