@@ -14,8 +14,8 @@
 
 #define MAX_STREAMS 8
 
-template <typename TO, int S, int VEC>
-__global__ __launch_bounds__(256) void hyper_norm_kernel(
+template <typename TO, int S, int VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void hyper_norm_kernel(
     float* __restrict__ streams, long long stream_stride, const float* __restrict__ update, int parts,
     long long part_stride, const float* __restrict__ mix, const float* __restrict__ share,
     const float* __restrict__ read, const float* __restrict__ weight, const float* __restrict__ bias, float eps,
@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
     for (int t = 0; t < S; ++t) m[s][t] = mix ? mix[s * S + t] : (s == t ? 1.f : 0.f);
   }
   float total = 0.f;
-  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+  for (int c = tid * VEC; c < W; c += THREADS * VEC) {
     float x[S][VEC], y[VEC];
 #pragma unroll
     for (int s = 0; s < S; ++s) {
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
   // a thread reads back only what it wrote itself: no barrier is needed before the passes below
   const float mean = rms ? 0.f : block_sum<true>(total, scratch) / (float)W;
   float squares = 0.f;
-  for (int c = tid * VEC; c < W; c += 256 * VEC)
+  for (int c = tid * VEC; c < W; c += THREADS * VEC)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       const float d = u_row[c + i] - mean;
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
   const float variance = block_sum(squares, scratch) / (float)W;
   const float inv = 1.f / sqrtf(variance + eps);
   TO* orow = out + (size_t)blockIdx.x * W;
-  for (int c = tid * VEC; c < W; c += 256 * VEC)
+  for (int c = tid * VEC; c < W; c += THREADS * VEC)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       float v = (u_row[c + i] - mean) * inv * weight[c + i];
@@ -119,12 +119,16 @@ static void launch_hyper(float* streams, long long stream_stride, const float* u
   const size_t lds = out ? (size_t)W * sizeof(float) : 0;
   const bool vec = W % 4 == 0 && ((uintptr_t)streams % 16 == 0) && stream_stride % 4 == 0 &&
                    (!update || ((uintptr_t)update % 16 == 0 && part_stride % 4 == 0));
-  if (vec)
-    hyper_norm_kernel<TO, S, 4><<<n_rows, 256, lds, stream>>>(streams, stream_stride, update, parts, part_stride, mix, share,
-                                                              read, weight, bias, eps, rms, (TO*)out, rows, W, store);
+  // a step of few rows is a matter of round trips, not of bytes: more threads a row then (one round of loads a thread)
+  if (vec && n_rows <= 512 && W >= 2048)
+    hyper_norm_kernel<TO, S, 4, 1024><<<n_rows, 1024, lds, stream>>>(streams, stream_stride, update, parts, part_stride, mix,
+                                                                     share, read, weight, bias, eps, rms, (TO*)out, rows, W, store);
+  else if (vec)
+    hyper_norm_kernel<TO, S, 4, 256><<<n_rows, 256, lds, stream>>>(streams, stream_stride, update, parts, part_stride, mix, share,
+                                                                   read, weight, bias, eps, rms, (TO*)out, rows, W, store);
   else
-    hyper_norm_kernel<TO, S, 1><<<n_rows, 256, lds, stream>>>(streams, stream_stride, update, parts, part_stride, mix, share,
-                                                              read, weight, bias, eps, rms, (TO*)out, rows, W, store);
+    hyper_norm_kernel<TO, S, 1, 256><<<n_rows, 256, lds, stream>>>(streams, stream_stride, update, parts, part_stride, mix, share,
+                                                                   read, weight, bias, eps, rms, (TO*)out, rows, W, store);
 }
 
 template <typename TO>

@@ -228,32 +228,52 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 #define TK 32
 #define TPAD 40
 
-template <int MODE>
+template <int MODE, int NT>
 __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
     const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
     float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
-    const float* __restrict__ extra, int extra_parts) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][TM][TPAD];
-  __shared__ int pair_of[TM];
+    const float* __restrict__ extra, int extra_parts, int slots, int column_tiles) {
+  // NT: groups of 16 columns a wave (a block takes 64 NT columns): with two, a fragment of rows read from LDS
+  // feeds twice the products, which is what a step of many rows is short of; a step of few rows takes one, for
+  // twice the blocks.  (Blocks of eight waves over 128 rows, the second four asking for the weight fragments of
+  // the first four, were measured slower: a prompt of 2,048 tokens 3.8 -> 4.3 ms at a width of 2,048.)
+  constexpr int ROWS = TM;
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][ROWS][TPAD];
+  __shared__ int pair_of[ROWS];
+  // Blocks go to the eight dies (XCDs, each with an L2 of its own) in turn by their index.  The row tiles of
+  // one expert under one column tile read the same part of the weight, so they are made neighbours in the
+  // order of work (the row slot runs fastest) and a die takes a run of that order: block b works on item
+  // (b % 8) * ceil(items / 8) + b / 8, and a weight tile comes from memory once for all its row tiles.
+  const int items = slots * column_tiles;
+  const int per_die = (items + 7) / 8;
+  const int item = (int)(blockIdx.x % 8) * per_die + (int)(blockIdx.x / 8);
+  if (item >= items) return;
   int expert, row0, row_end;
-  if (!find_tile<TM>(offsets, E, blockIdx.x, expert, row0, row_end)) return;
+  if (!find_tile<ROWS>(offsets, E, item % slots, expert, row0, row_end)) return;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 16, lq = lane / 16;
-  const int n0 = blockIdx.y * TN;
-  if (tid < TM) pair_of[tid] = row0 + tid < row_end ? order[row0 + tid] : -1;
+  const int n0 = (item / slots) * (TN * NT);
+  if (tid < ROWS) pair_of[tid] = row0 + tid < row_end ? order[row0 + tid] : -1;
   __syncthreads();
   // this thread's 16 bytes of a step's rows: row tid / 4, k chunk tid % 4
   const int my_row = tid / 4, my_chunk = tid % 4;
   const int my_pair = pair_of[my_row];
   const size_t src = my_pair < 0 ? 0 : (MODE == 0 ? (size_t)(my_pair / top) : (size_t)(row0 + my_row));
   const bf16_t* a_at = a + src * K + my_chunk * 8;
-  const int n = n0 + wave * 16 + lr;
   const size_t w_rows = MODE == 0 ? 2 * (size_t)N : (size_t)N;
-  const bf16_t* wg_at = w + ((size_t)expert * w_rows + min(n, N - 1)) * K + lq * 8;
-  const bf16_t* wu_at = wg_at + (MODE == 0 ? (size_t)N * K : 0);
-  floatx4 acc_g[4], acc_u[4];
+  int n[NT];
+  const bf16_t* wg_at[NT];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) acc_g[mt] = acc_u[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int nt = 0; nt < NT; ++nt) {
+    n[nt] = n0 + (wave * NT + nt) * 16 + lr;
+    wg_at[nt] = w + ((size_t)expert * w_rows + min(n[nt], N - 1)) * K + lq * 8;
+  }
+  const size_t up_offset = MODE == 0 ? (size_t)N * K : 0;
+  floatx4 acc_g[NT][4], acc_u[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc_g[nt][mt] = acc_u[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const uintx4 zero = {0u, 0u, 0u, 0u};
   // Step s has its operands in register set s % DEPTH, requested DEPTH steps ahead (a step's arithmetic is far
   // shorter than a trip to memory, and a launch of few blocks keeps the memory busy only through what each
@@ -262,20 +282,26 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
   // step's operands again, so that no load stands under a branch.
   constexpr int DEPTH = 4;
   const int steps = K / TK;
-  uintx4 a_reg[DEPTH], wg_reg[DEPTH], wu_reg[DEPTH];
+  uintx4 a_reg[DEPTH], wg_reg[DEPTH][NT], wu_reg[DEPTH][NT];
   auto fetch = [&](int step, int set) {
     const int at = min(step, steps - 1) * TK;
     a_reg[set] = *(const uintx4*)(a_at + at);
-    wg_reg[set] = *(const uintx4*)(wg_at + at);
-    if (MODE == 0) wu_reg[set] = *(const uintx4*)(wu_at + at);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      wg_reg[set][nt] = *(const uintx4*)(wg_at[nt] + at);
+      if (MODE == 0) wu_reg[set][nt] = *(const uintx4*)(wg_at[nt] + up_offset + at);
+    }
   };
   auto multiply = [&](int stage, int set) {
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       const bf16x8 rows = *(const bf16x8*)&As[stage][mt * 16 + lr][lq * 8];
-      acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wg_reg[set]), acc_g[mt], 0, 0, 0);
-      if (MODE == 0)
-        acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wu_reg[set]), acc_u[mt], 0, 0, 0);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        acc_g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wg_reg[set][nt]), acc_g[nt][mt], 0, 0, 0);
+        if (MODE == 0)
+          acc_u[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, __builtin_bit_cast(bf16x8, wu_reg[set][nt]), acc_u[nt][mt], 0, 0, 0);
+      }
     }
   };
   auto stash = [&](int stage, int set) { *(uintx4*)&As[stage][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_reg[set]; };
@@ -301,23 +327,46 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
       stash((u + 1) & 1, (u + 1) % DEPTH);
       __syncthreads();
     }
-  if (n >= N) return;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int nt = 0; nt < NT; ++nt) {
+    if (n[nt] >= N) continue;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = mt * 16 + lq * 4 + i;
-      const int pair = pair_of[r];
-      if (pair < 0) continue;
-      if (MODE == 0) {
-        act[(size_t)(row0 + r) * N + n] = float_to_bf16(gated(acc_g[mt][i], acc_u[mt][i], limit, alpha));
-      } else {
-        const int token = pair / top, choice = pair - token * top;
-        out[((size_t)choice * tokens + token) * N + n] =
-            with_extra(acc_g[mt][i] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = mt * 16 + lq * 4 + i;
+        const int pair = pair_of[r];
+        if (pair < 0) continue;
+        if (MODE == 0) {
+          act[(size_t)(row0 + r) * N + n[nt]] = float_to_bf16(gated(acc_g[nt][mt][i], acc_u[nt][mt][i], limit, alpha));
+        } else {
+          const int token = pair / top, choice = pair - token * top;
+          out[((size_t)choice * tokens + token) * N + n[nt]] = with_extra(
+              acc_g[nt][mt][i] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n[nt]);
+        }
       }
-    }
+  }
 }
+
+// Two groups of columns a wave from this many pairs on (the launch then still has blocks enough).
+#define WIDE_COLUMNS_MIN_PAIRS 1024
+
+// blocks of a launch: the items rounded up to a whole number a die
+static unsigned mfma_blocks(int slots, int column_tiles) { return (unsigned)(((long long)slots * column_tiles + 7) / 8 * 8); }
+
+// Which shape a launch takes: two column groups a wave from WIDE_COLUMNS_MIN_PAIRS pairs on.
+#define MFMA_LAUNCH(MODE, COLUMNS, A, W, PW, ACT, OUT, N_, K_, LIMIT, ALPHA, EXTRA, EXTRA_PARTS)                          \
+  do {                                                                                                                   \
+    const bool wide = pairs >= WIDE_COLUMNS_MIN_PAIRS;                                                                   \
+    const int slots = (int)(pairs / TM + experts);                                                                       \
+    const int tiles = ((COLUMNS) + (wide ? 2 : 1) * TN - 1) / ((wide ? 2 : 1) * TN);                                      \
+    if (wide)                                                                                                            \
+      moe_grouped_mfma_kernel<MODE, 2><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                   \
+          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
+    else                                                                                                                 \
+      moe_grouped_mfma_kernel<MODE, 1><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                   \
+          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
+  } while (0)
 
 static bool mfma_fits(const void* a, const void* w, int K) {
   return K % TK == 0 && ((((uintptr_t)a) | ((uintptr_t)w)) & 15) == 0;
@@ -333,11 +382,9 @@ extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, con
   if (dtype == FE_F32)
     moe_grouped_kernel<float, 0><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, offsets, order, nullptr,
                                                            (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha, nullptr, 0);
-  else if (dtype == FE_BF16 && mfma_fits(x, gate_up, hidden))
-    moe_grouped_mfma_kernel<0><<<dim3((unsigned)(pairs / TM + experts), (unsigned)((inner + TN - 1) / TN)), 256, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr, (bf16_t*)act, nullptr, experts, inner, hidden, top,
-        tokens, limit, alpha, nullptr, 0);
-  else if (dtype == FE_BF16)
+  else if (dtype == FE_BF16 && mfma_fits(x, gate_up, hidden)) {
+    MFMA_LAUNCH(0, inner, (const bf16_t*)x, (const bf16_t*)gate_up, nullptr, (bf16_t*)act, nullptr, inner, hidden, limit, alpha, nullptr, 0);
+  } else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr,
                                                             (bf16_t*)act, nullptr, experts, inner, hidden, top, tokens, limit,
                                                             alpha, nullptr, 0);
@@ -357,11 +404,9 @@ extern "C" int fe_moe_down(const void* act, const void* down, int dtype, const i
     moe_grouped_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, offsets, order, pair_weight,
                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, extra,
                                                            extra_parts);
-  else if (dtype == FE_BF16 && mfma_fits(act, down, inner))
-    moe_grouped_mfma_kernel<1><<<dim3((unsigned)(pairs / TM + experts), (unsigned)((hidden + TN - 1) / TN)), 256, 0, stream>>>(
-        (const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight, nullptr, out, experts, hidden, inner, top, tokens,
-        0.f, 0.f, extra, extra_parts);
-  else if (dtype == FE_BF16)
+  else if (dtype == FE_BF16 && mfma_fits(act, down, inner)) {
+    MFMA_LAUNCH(1, hidden, (const bf16_t*)act, (const bf16_t*)down, pair_weight, nullptr, out, hidden, inner, 0.f, 0.f, extra, extra_parts);
+  } else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight,
                                                             nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, extra,
                                                            extra_parts);

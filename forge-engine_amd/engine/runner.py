@@ -296,6 +296,12 @@ class ModelRunner:
         states = self.embedding_states
         return CacheView(states={name: state.clone() for name, state in states.items()} if scratch_state else states)
 
+    def _forward(self, batch: StepBatch, views, scratch_state: bool = False) -> Tensor:
+        """The model's forward pass over the step's batch; an embedding that keeps state gets its view."""
+        if not self.embedding_states:
+            return self.model.forward(batch, views)
+        return self.model.forward(batch, views, self.embedding_view(scratch_state))
+
     def _graphable(self, entries: list[StepEntry]) -> bool:
         return (self.use_graphs and len(entries) <= GRAPH_MAX_REQUESTS
                 and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
@@ -372,7 +378,7 @@ class ModelRunner:
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                slot.logits = self.model.forward(batch, views, self.embedding_view())
+                slot.logits = self._forward(batch, views)
             slot.graph, slot.views, slot.batch = graph, views, batch
         if device_tokens is not None:
             slot.feed(device_tokens)
@@ -394,7 +400,7 @@ class ModelRunner:
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(side):
-            self.model.forward(batch, views, self.embedding_view(scratch_state=True))
+            self._forward(batch, views, scratch_state=True)
         torch.cuda.current_stream(self.device).wait_stream(side)
 
     def _portion_key(self, entries: list[StepEntry]):
@@ -453,7 +459,7 @@ class ModelRunner:
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                slot.logits = self.model.forward(batch, views, self.embedding_view())
+                slot.logits = self._forward(batch, views)
             slot.graph, slot.views, slot.batch = graph, views, batch
         slot.graph.replay()
         self.portion_graph_replays += 1
@@ -496,7 +502,7 @@ class ModelRunner:
             if logits is not None:
                 return logits
         batch = self.prepare(entries)
-        logits = self.model.forward(batch, self.cache_views(batch), self.embedding_view())
+        logits = self._forward(batch, self.cache_views(batch))
         for i, entry in enumerate(entries):
             self.cache.commit(entry.request_id, batch.ctx_before_host[i] + batch.q_lens[i])
         self.steps_run += 1

@@ -123,11 +123,11 @@ class GroupedQueryAttention(Mixer):
         n = {key: self.name(leaf) for key, leaf in self.names.items()}
         specs = {
             n["q"]: ParamSpec((self.q_size, self.hidden_size)),
-            n["o"]: ParamSpec((self.hidden_size, self.out_size)),
         }
         if self.own_kv:
             specs[n["k"]] = ParamSpec((self.kv_size, self.hidden_size))
             specs[n["v"]] = ParamSpec((self.v_size, self.hidden_size))
+        specs[n["o"]] = ParamSpec((self.hidden_size, self.out_size))
         if self.whole_norm_eps is not None:
             specs[n["q_norm"]] = ParamSpec((self.q_size,), kind="vector", init="norm")
             if self.own_kv:

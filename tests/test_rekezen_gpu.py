@@ -211,3 +211,176 @@ def test_replay_matches_plain(name, mode, dtype, folders, plain_cache, tmp_path)
     got = ru.run_trace(folders[name], dtype, trace, tmp_path, block_size=BLOCKS[name])
     worst = ku.compare(got, expected(name, folders[name], plain_cache, requests), dtype)
     print(f"  worst difference {worst:.3e}", flush=True)
+
+
+def sharp(folder, target, factor=6.0):
+    """A copy of a model whose attention is sharp (larger norm weights on q, no cap below the scores'
+    range), so that one key among hundreds, however far back, moves the logits."""
+    import json
+    from safetensors.torch import save_file
+    raw, weights = ku.folder_weights(folder)
+    for index, layer in enumerate(raw["layers"]):
+        weights[f"l{index}.mix.q.norm"] = weights[f"l{index}.mix.q.norm"] * factor
+        if "softcap" in layer["mixer"]:
+            layer["mixer"]["softcap"] = 40.0
+    target.mkdir(parents=True, exist_ok=True)
+    (target / "config.json").write_text(json.dumps(raw))
+    save_file({n: t.contiguous() for n, t in weights.items()}, str(target / "model.safetensors"))
+    return target
+
+
+def test_far_tokens_reach_the_logits(folders, tmp_path):
+    """A control on the weights made above: with them, changing the third token of 500 changes the
+    last token's logits by more than the float32 bound of these tests."""
+    folder = sharp(folders["M"], tmp_path / "sharp")
+    cfg, weights = ku.folder_weights(folder)
+    tokens = requests_of("M", 8, (500,))["r0"]
+    other = list(tokens)
+    other[2] = (other[2] + 1) % cfg["vocab"]
+    a, b = ku.plain.forward(tokens, weights, cfg)[-1], ku.plain.forward(other, weights, cfg)[-1]
+    assert float((a - b).abs().max()) > 1000 * (1e-5 + 1e-4 * float(a.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_requests_with_sharp_attention(dtype, folders, tmp_path):
+    """Prompts of several hundred tokens whose far keys matter: whole, then the last 40 tokens one by
+    one (across page borders), then in portions, then three at once."""
+    folder = sharp(folders["M"], tmp_path / "sharp")
+    requests = requests_of("M", 9, (500, 333, 129))
+    want = ku.plain_logits(folder, requests)
+    for mode, trace in (("whole", ru.trace_whole(requests)), ("tail", ru.trace_tail(requests, 40)),
+                        ("portions", ru.trace_portions(requests, sizes=(64, 17, 2, 130, 3, 48, 16, 2, 33), want_all=False)),
+                        ("mixed", ru.trace_mixed(requests, 11, max_live=3))):
+        print(f"sharp {mode} {dtype}: {len(trace.steps)} steps", flush=True)
+        got = ru.run_trace(folder, dtype, trace, tmp_path / mode, block_size=16)
+        # scores of up to 40 turn an error of one part in 10**7 in a key into one of some parts in 10**5 in a
+        # softmax weight: float32 differs from the plain implementation by up to 1e-4 here (the plain
+        # implementation in float32 does too); a key left out moves these logits by a hundred times that
+        ku.compare(got, want, dtype, fraction=0.1, float32_factor=10.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("block_size", [4, 16, 32])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 32, 16), (6, 3, 64, 64), (8, 1, 128, 128)])
+def test_one_far_key_among_hundreds_is_found(dtype, block_size, heads, kv_heads, dim, vdim):
+    """Keys whose scores dominate sit at the first position, just before and at page borders and hundreds
+    of positions back: the attention kernels (matrix cores for heads of 64 and 128 in bfloat16 with pages
+    of 16 or more, the vector ALU otherwise) against the plain capped attention, for a prompt's portion
+    behind cached keys and for single tokens; with a cap that the dominant scores reach."""
+    from forge_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(dim + block_size)
+    length, cached = 420, 391          # the portion's 29 tokens lie behind 391 cached ones
+    q = torch.randn(length, heads, dim, generator=g)
+    k = torch.randn(length, kv_heads, dim, generator=g)
+    v = torch.randn(length, kv_heads, vdim, generator=g)
+    for far in (0, block_size - 1, block_size, 7 * block_size - 1, 7 * block_size, 200, cached - 1, cached):
+        k[far] *= 5.0
+    q, k, v = (t.to(dtype) for t in (q, k, v))
+    cap, scale = 9.0, 0.3
+    want = ku.plain.capped_causal_attention(q.double(), k.double(), v.double(), scale=scale, softcap=cap)
+    gates = torch.randn(length, heads, generator=g).to(dtype)
+    want = (want * torch.sigmoid(gates.double())[:, :, None]).reshape(length, heads * vdim).float()
+    pages = -(-length // block_size)
+    perm = torch.randperm(pages + 3, generator=g)[:pages].to(torch.int32)
+    key_pages = torch.zeros(pages + 3, kv_heads, block_size, dim, dtype=dtype)
+    value_pages = torch.zeros(pages + 3, kv_heads, vdim, block_size, dtype=dtype)
+    for p in range(length):
+        key_pages[perm[p // block_size], :, p % block_size] = k[p]
+        value_pages[perm[p // block_size], :, :, p % block_size] = v[p]
+    key_pages, value_pages = key_pages.to(DEV), value_pages.to(DEV)
+    table = perm.view(1, -1).to(DEV)
+    common = dict(q_heads=heads, kv_heads=kv_heads, head_dim=dim, value_dim=vdim, scale=scale, softcap=cap, head_gate=True)
+    # the portion
+    out = torch.empty(length - cached, heads * vdim, dtype=dtype, device=DEV)
+    ops.masked_attention(q[cached:].reshape(length - cached, -1).to(DEV), key_pages, value_pages, out,
+                         torch.tensor([0, length - cached], dtype=torch.int32, device=DEV), torch.tensor([length], dtype=torch.int32, device=DEV),
+                         table, num_seqs=1, max_q_len=length - cached, gate=gates[cached:].to(DEV), num_decode=0, max_ctx=length, **common)
+    close(out, want[cached:], dtype)
+    # single tokens: the same request at eight of its lengths, as eight sequences of one step
+    places = [0, block_size - 1, block_size, 7 * block_size, 201, cached - 1, cached, length - 1]
+    n = len(places)
+    out = torch.empty(n, heads * vdim, dtype=dtype, device=DEV)
+    ops.masked_attention(q[places].reshape(n, -1).to(DEV), key_pages, value_pages, out,
+                         torch.arange(n + 1, dtype=torch.int32, device=DEV), torch.tensor([p + 1 for p in places], dtype=torch.int32, device=DEV),
+                         table.expand(n, -1).contiguous(), num_seqs=n, max_q_len=1, gate=gates[places].to(DEV), num_decode=n,
+                         max_ctx=length, **common)
+    close(out, want[places], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_steps_equal_eager_steps_and_long_decoding(dtype, folders):
+    """A prompt and then 150 single tokens, two requests side by side: steps replayed from captured graphs
+    against the same steps run eagerly, and both against the plain implementation."""
+    from forge_engine_amd.engine import ModelRunner, StepEntry, load_model
+    _, model = load_model(folders["M"], dtype=dtype, device=DEV)
+    requests = requests_of("M", 21, (160, 171))
+    want = ku.plain_logits(folders["M"], requests)
+    results = {}
+    for graphs in (True, False):
+        runner = ModelRunner(model, block_size=16, block_capacity=40, num_state_slots=3, use_graphs=graphs, eager_sightings=1)
+        got = {}
+        for name in requests:
+            runner.begin(name)
+        at = {"r0": 10, "r1": 21}
+        logits = runner.step([StepEntry(n, requests[n][:at[n]], [at[n] - 1]) for n in requests])
+        for row, n in zip(logits, requests):
+            got[(n, at[n] - 1)] = row.cpu().clone()
+        for _ in range(150):
+            logits = runner.step([StepEntry(n, [requests[n][at[n]]], [0]) for n in requests])
+            for row, n in zip(logits, requests):
+                got[(n, at[n])] = row.cpu().clone()
+                at[n] += 1
+        assert runner.graph_replays >= (140 if graphs else 0) and (graphs or runner.graph_replays == 0)
+        results[graphs] = got
+        ku.compare(got, want, dtype, fraction=0.1)
+    for key, row in results[True].items():
+        torch.testing.assert_close(row, results[False][key], rtol=0, atol=0 if dtype == "float32" else 1e-2)
+
+
+def test_first_tokens_and_slot_reuse(folders):
+    """A request that takes over the state slot of one that ended: its first token has no token before
+    it, whatever the slot still holds; requests of one and two tokens."""
+    from forge_engine_amd.engine import ModelRunner, StepEntry, load_model
+    _, model = load_model(folders["A"], dtype="float32", device=DEV)
+    runner = ModelRunner(model, block_size=4, block_capacity=16, num_state_slots=1)
+    cfg, weights = ku.folder_weights(folders["A"])
+    for tokens in ([5, 90, 17, 3], [44], [7, 7], [90, 5, 17, 3, 3, 3, 8, 1, 2]):
+        runner.begin("only")
+        rows = []
+        for token in tokens:          # token by token: every token's predecessor comes from the slot
+            rows.append(runner.step([StepEntry("only", [token], [0])])[0].cpu().clone())
+        runner.end("only")
+        want = ku.plain.forward(tokens, weights, cfg)
+        for got, expected in zip(rows, want):
+            assert float((got.double() - expected).abs().max()) <= 1e-5 + 1e-4 * float(expected.abs().max())
+
+
+def test_generation_through_the_entry_point_and_the_command_line(folders):
+    import os
+    import subprocess
+    import sys
+    from conftest import ROOT
+    from forge_engine_amd.config import SchedulerConfig
+    from forge_engine_amd.engine import engine_from_folder
+    from forge_engine_amd.sampling import SamplingParams
+
+    cfg, weights = ku.folder_weights(folders["A"])
+
+    def greedy(prompt, count):
+        tokens = list(prompt)
+        for _ in range(count):
+            tokens.append(int(ku.plain.forward(tokens, weights, cfg)[-1].argmax()))
+        return tokens[len(prompt):]
+
+    prompts = list(requests_of("A", 13, (11, 3, 25)).values())
+    want = [greedy(prompt, 8) for prompt in prompts]
+    engine = engine_from_folder(folders["A"], scheduler_config=SchedulerConfig(block_size=4, block_capacity=128, token_budget=16),
+                                dtype="float32", eos_token_ids=[])
+    ids = [engine.submit(prompt, sampling_params=SamplingParams(max_new_tokens=8)) for prompt in prompts]
+    engine.run_until_idle()
+    assert [list(engine.request(i).output_token_ids) for i in ids] == want
+    command = [sys.executable, str(ROOT / "bin" / "forge-engine"), "generate", "--model", str(folders["A"]), "--dtype", "float32",
+               "--max-new-tokens", "8", "--block-size", "4", "--prompt-ids", ",".join(map(str, prompts[0]))]
+    done = subprocess.run(command, capture_output=True, text=True, timeout=300, env=dict(os.environ))
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert ",".join(map(str, want[0])) in done.stdout.replace(" ", "")
