@@ -228,17 +228,30 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 #define TK 32
 #define TPAD 40
 
-template <int MODE, int NT>
+// A barrier that orders the block's LDS traffic only: the loads from global memory that are under way for
+// later steps stay under way (a barrier that fences every address space waits for all of them, and the
+// operands requested steps ahead would arrive no earlier than those of the step at hand).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int MODE, int NT, int MT>
 __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
     const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
     float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
     const float* __restrict__ extra, int extra_parts, int slots, int column_tiles) {
-  // NT: groups of 16 columns a wave (a block takes 64 NT columns): with two, a fragment of rows read from LDS
-  // feeds twice the products, which is what a step of many rows is short of; a step of few rows takes one, for
-  // twice the blocks.  (Blocks of eight waves over 128 rows, the second four asking for the weight fragments of
-  // the first four, were measured slower: a prompt of 2,048 tokens 3.8 -> 4.3 ms at a width of 2,048.)
-  constexpr int ROWS = TM;
+  // NT: groups of 16 columns a wave (a block takes 64 NT columns); MT: tiles of 16 rows a wave (a block takes
+  // 16 MT rows, every wave all of them).  What bounds a step of many rows is what crosses from the L2 to the
+  // CUs: a block of 64 x 128 pulls 19 bytes for every thousand multiply-adds, one of 128 x 128 eleven, and a
+  // fragment of rows read from LDS feeds NT products, a fragment of the weight MT.  A step of few rows takes
+  // the small shape, for more blocks.  (Blocks of eight waves over 128 rows, the second four asking for the
+  // weight fragments of the first four, were measured slower: a prompt of 2,048 tokens 3.8 -> 4.3 ms at a
+  // width of 2,048; the L1 does not hold what the other wave asked for.)
+  constexpr int ROWS = 16 * MT;
+  constexpr int AL = ROWS / 64;          // 16-byte pieces of a step's rows a thread brings
   __shared__ __attribute__((aligned(16))) bf16_t As[2][ROWS][TPAD];
   __shared__ int pair_of[ROWS];
   // Blocks go to the eight dies (XCDs, each with an L2 of its own) in turn by their index.  The row tiles of
@@ -253,13 +266,21 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
   if (!find_tile<ROWS>(offsets, E, item % slots, expert, row0, row_end)) return;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 16, lq = lane / 16;
   const int n0 = (item / slots) * (TN * NT);
-  if (tid < ROWS) pair_of[tid] = row0 + tid < row_end ? order[row0 + tid] : -1;
+  for (int r = tid; r < ROWS; r += 256) pair_of[r] = row0 + r < row_end ? order[row0 + r] : -1;
   __syncthreads();
-  // this thread's 16 bytes of a step's rows: row tid / 4, k chunk tid % 4
-  const int my_row = tid / 4, my_chunk = tid % 4;
-  const int my_pair = pair_of[my_row];
-  const size_t src = my_pair < 0 ? 0 : (MODE == 0 ? (size_t)(my_pair / top) : (size_t)(row0 + my_row));
-  const bf16_t* a_at = a + src * K + my_chunk * 8;
+  // this thread's 16-byte pieces of a step's rows: rows tid / 4 + 64 j, k chunk tid % 4
+  const int my_chunk = tid % 4;
+  int my_row[AL];
+  bool my_live[AL];
+  const bf16_t* a_at[AL];
+#pragma unroll
+  for (int j = 0; j < AL; ++j) {
+    my_row[j] = tid / 4 + 64 * j;
+    const int pair = pair_of[my_row[j]];
+    my_live[j] = pair >= 0;
+    const size_t src = pair < 0 ? 0 : (MODE == 0 ? (size_t)(pair / top) : (size_t)(row0 + my_row[j]));
+    a_at[j] = a + src * K + my_chunk * 8;
+  }
   const size_t w_rows = MODE == 0 ? 2 * (size_t)N : (size_t)N;
   int n[NT];
   const bf16_t* wg_at[NT];
@@ -269,23 +290,24 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     wg_at[nt] = w + ((size_t)expert * w_rows + min(n[nt], N - 1)) * K + lq * 8;
   }
   const size_t up_offset = MODE == 0 ? (size_t)N * K : 0;
-  floatx4 acc_g[NT][4], acc_u[NT][4];
+  floatx4 acc_g[NT][MT], acc_u[NT][MT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc_g[nt][mt] = acc_u[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt) acc_g[nt][mt] = acc_u[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const uintx4 zero = {0u, 0u, 0u, 0u};
   // Step s has its operands in register set s % DEPTH, requested DEPTH steps ahead (a step's arithmetic is far
   // shorter than a trip to memory, and a launch of few blocks keeps the memory busy only through what each
   // block has in flight).  The rows of step s + 1 go into the other LDS stage while step s multiplies; one
   // barrier a step.  Whole rounds of DEPTH steps are straight-line code; steps beyond the last fetch the last
   // step's operands again, so that no load stands under a branch.
-  constexpr int DEPTH = 4;
+  constexpr int DEPTH = MT > 4 ? 2 : 4;
   const int steps = K / TK;
-  uintx4 a_reg[DEPTH], wg_reg[DEPTH][NT], wu_reg[DEPTH][NT];
+  uintx4 a_reg[DEPTH][AL], wg_reg[DEPTH][NT], wu_reg[DEPTH][NT];
   auto fetch = [&](int step, int set) {
     const int at = min(step, steps - 1) * TK;
-    a_reg[set] = *(const uintx4*)(a_at + at);
+#pragma unroll
+    for (int j = 0; j < AL; ++j) a_reg[set][j] = *(const uintx4*)(a_at[j] + at);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       wg_reg[set][nt] = *(const uintx4*)(wg_at[nt] + at);
@@ -294,7 +316,7 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
   };
   auto multiply = [&](int stage, int set) {
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const bf16x8 rows = *(const bf16x8*)&As[stage][mt * 16 + lr][lq * 8];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
@@ -304,11 +326,14 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
       }
     }
   };
-  auto stash = [&](int stage, int set) { *(uintx4*)&As[stage][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_reg[set]; };
+  auto stash = [&](int stage, int set) {
+#pragma unroll
+    for (int j = 0; j < AL; ++j) *(uintx4*)&As[stage][my_row[j]][my_chunk * 8] = my_live[j] ? a_reg[set][j] : zero;
+  };
 #pragma unroll
   for (int u = 0; u < DEPTH; ++u) fetch(u, u);
   stash(0, 0);
-  __syncthreads();
+  lds_barrier();
   int step = 0;
   for (; step + DEPTH <= steps; step += DEPTH) {
 #pragma unroll
@@ -316,7 +341,7 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
       multiply(u & 1, u);
       stash((u + 1) & 1, (u + 1) % DEPTH);
       fetch(step + u + DEPTH, u);
-      __syncthreads();
+      lds_barrier();
     }
   }
   const int left = steps - step;       // 0 .. DEPTH - 1, the same for every thread
@@ -325,13 +350,13 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     if (u < left) {
       multiply(u & 1, u);
       stash((u + 1) & 1, (u + 1) % DEPTH);
-      __syncthreads();
+      lds_barrier();
     }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     if (n[nt] >= N) continue;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = mt * 16 + lq * 4 + i;
@@ -354,17 +379,22 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
 // blocks of a launch: the items rounded up to a whole number a die
 static unsigned mfma_blocks(int slots, int column_tiles) { return (unsigned)(((long long)slots * column_tiles + 7) / 8 * 8); }
 
-// Which shape a launch takes: two column groups a wave from WIDE_COLUMNS_MIN_PAIRS pairs on.
+// Which shape a launch takes: two column groups a wave from WIDE_COLUMNS_MIN_PAIRS pairs on, and blocks of 128
+// rows where an expert has at least two such tiles on average and K is 4,096 or more (measured, a prompt of
+// 2,048 tokens: at a width of 4,096 10.0 -> 9.7 ms, at 2,048 3.80 -> 3.89 ms).
 #define MFMA_LAUNCH(MODE, COLUMNS, A, W, PW, ACT, OUT, N_, K_, LIMIT, ALPHA, EXTRA, EXTRA_PARTS)                          \
   do {                                                                                                                   \
-    const bool wide = pairs >= WIDE_COLUMNS_MIN_PAIRS;                                                                   \
-    const int slots = (int)(pairs / TM + experts);                                                                       \
+    const bool wide = pairs >= WIDE_COLUMNS_MIN_PAIRS, tall = wide && pairs / experts >= 256 && (K_) >= 4096;                             \
+    const int slots = (int)(pairs / (tall ? 128 : TM) + experts);                                                        \
     const int tiles = ((COLUMNS) + (wide ? 2 : 1) * TN - 1) / ((wide ? 2 : 1) * TN);                                      \
-    if (wide)                                                                                                            \
-      moe_grouped_mfma_kernel<MODE, 2><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                   \
+    if (tall)                                                                                                            \
+      moe_grouped_mfma_kernel<MODE, 2, 8><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \
+          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
+    else if (wide)                                                                                                       \
+      moe_grouped_mfma_kernel<MODE, 2, 4><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \
           A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
     else                                                                                                                 \
-      moe_grouped_mfma_kernel<MODE, 1><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                   \
+      moe_grouped_mfma_kernel<MODE, 1, 4><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \
           A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
   } while (0)
 
