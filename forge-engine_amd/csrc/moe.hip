@@ -244,12 +244,11 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
     const float* __restrict__ extra, int extra_parts, int slots, int column_tiles) {
   // NT: groups of 16 columns a wave (a block takes 64 NT columns); MT: tiles of 16 rows a wave (a block takes
-  // 16 MT rows, every wave all of them).  What bounds a step of many rows is what crosses from the L2 to the
-  // CUs: a block of 64 x 128 pulls 19 bytes for every thousand multiply-adds, one of 128 x 128 eleven, and a
-  // fragment of rows read from LDS feeds NT products, a fragment of the weight MT.  A step of few rows takes
-  // the small shape, for more blocks.  (Blocks of eight waves over 128 rows, the second four asking for the
-  // weight fragments of the first four, were measured slower: a prompt of 2,048 tokens 3.8 -> 4.3 ms at a
-  // width of 2,048; the L1 does not hold what the other wave asked for.)
+  // 16 MT rows, every wave all of them).  Steps of few rows launch <MODE, 1, 4>: many blocks, each streaming
+  // its part of the weight.  For steps of many rows the larger shapes of this kernel were measured and lost to
+  // the kernel below, whose weight tile goes through LDS (<MODE, 2, 4>: 3.80 against 3.67 ms for a prompt of 2,048
+  // tokens at a width of 2,048; <MODE, 2, 8> at 4,096: 9.9 against 9.6 ms; eight waves over 128 rows, the second
+  // four asking for the weight fragments of the first four: 4.3 ms at 2,048).
   constexpr int ROWS = 16 * MT;
   constexpr int AL = ROWS / 64;          // 16-byte pieces of a step's rows a thread brings
   __shared__ __attribute__((aligned(16))) bf16_t As[2][ROWS][TPAD];
@@ -373,25 +372,148 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
   }
 }
 
+// The shape for steps of many rows: the weight tile goes through LDS as the rows do.  Straight into the MFMA
+// operand, a lane asks for 16 bytes of a weight row of its own, and the 64 lanes of a load are 64 accesses of
+// the CU's L1 (measured: 80 million a launch, 312,000 a CU in 473,000 cycles, with the matrix cores busy 14 %);
+// here four neighbouring lanes bring 64 neighbouring bytes of one weight row, a quarter of the accesses, and every
+// wave reads its fragments out of LDS.  Block = 64 rows x 128 columns (MODE 0: and their 128 up columns), K in
+// steps of 32, two stages, operands requested DEPTH steps ahead, one LDS-only barrier a step.
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_grouped_staged_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
+    const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
+    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
+    const float* __restrict__ extra, int extra_parts, int slots, int column_tiles) {
+  constexpr int COLS = 128, MATS = MODE == 0 ? 2 : 1, NT = 2, MT = 4;
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][TM][TPAD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][MATS][COLS][TPAD];
+  __shared__ int pair_of[TM];
+  const int items = slots * column_tiles;
+  const int per_die = (items + 7) / 8;
+  const int item = (int)(blockIdx.x % 8) * per_die + (int)(blockIdx.x / 8);
+  if (item >= items) return;
+  int expert, row0, row_end;
+  if (!find_tile<TM>(offsets, E, item % slots, expert, row0, row_end)) return;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 16, lq = lane / 16;
+  const int n0 = (item / slots) * COLS;
+  if (tid < TM) pair_of[tid] = row0 + tid < row_end ? order[row0 + tid] : -1;
+  __syncthreads();
+  // a thread's 16-byte pieces of a step: row tid / 4 of the rows, weight rows tid / 4 and tid / 4 + 64 of each
+  // matrix, k chunk tid % 4
+  const int my_row = tid / 4, my_chunk = tid % 4;
+  const int my_pair = pair_of[my_row];
+  const size_t src = my_pair < 0 ? 0 : (MODE == 0 ? (size_t)(my_pair / top) : (size_t)(row0 + my_row));
+  const bf16_t* a_at = a + src * K + my_chunk * 8;
+  const size_t w_rows = MODE == 0 ? 2 * (size_t)N : (size_t)N;
+  const bf16_t* w_at[MATS][2];
+#pragma unroll
+  for (int m = 0; m < MATS; ++m)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      w_at[m][j] = w + ((size_t)expert * w_rows + (size_t)m * N + min(n0 + my_row + 64 * j, N - 1)) * K + my_chunk * 8;
+  floatx4 acc[MATS][NT][MT];
+#pragma unroll
+  for (int m = 0; m < MATS; ++m)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[m][nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const uintx4 zero = {0u, 0u, 0u, 0u};
+  constexpr int DEPTH = MODE == 0 ? 2 : 4;      // with two matrices the registers hold two steps' operands beside the sums
+  const int steps = K / TK;
+  uintx4 a_reg[DEPTH], w_reg[DEPTH][MATS][2];
+  auto fetch = [&](int step, int set) {
+    const int at = min(step, steps - 1) * TK;
+    a_reg[set] = *(const uintx4*)(a_at + at);
+#pragma unroll
+    for (int m = 0; m < MATS; ++m)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) w_reg[set][m][j] = *(const uintx4*)(w_at[m][j] + at);
+  };
+  auto stash = [&](int stage, int set) {
+    *(uintx4*)&As[stage][my_row][my_chunk * 8] = my_pair < 0 ? zero : a_reg[set];
+#pragma unroll
+    for (int m = 0; m < MATS; ++m)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) *(uintx4*)&Ws[stage][m][my_row + 64 * j][my_chunk * 8] = w_reg[set][m][j];
+  };
+  auto multiply = [&](int stage) {
+    bf16x8 cols[MATS][NT];
+#pragma unroll
+    for (int m = 0; m < MATS; ++m)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) cols[m][nt] = *(const bf16x8*)&Ws[stage][m][(wave * NT + nt) * 16 + lr][lq * 8];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const bf16x8 rows = *(const bf16x8*)&As[stage][mt * 16 + lr][lq * 8];
+#pragma unroll
+      for (int m = 0; m < MATS; ++m)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[m][nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, cols[m][nt], acc[m][nt][mt], 0, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) fetch(u, u);
+  stash(0, 0);
+  lds_barrier();
+  int step = 0;
+  for (; step + DEPTH <= steps; step += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      multiply(u & 1);
+      stash((u + 1) & 1, (u + 1) % DEPTH);
+      fetch(step + u + DEPTH, u);
+      lds_barrier();
+    }
+  }
+  const int left = steps - step;
+#pragma unroll
+  for (int u = 0; u < DEPTH - 1; ++u)
+    if (u < left) {
+      multiply(u & 1);
+      stash((u + 1) & 1, (u + 1) % DEPTH);
+      lds_barrier();
+    }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = n0 + (wave * NT + nt) * 16 + lr;
+    if (n >= N) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = mt * 16 + lq * 4 + i;
+        const int pair = pair_of[r];
+        if (pair < 0) continue;
+        if (MODE == 0) {
+          act[(size_t)(row0 + r) * N + n] = float_to_bf16(gated(acc[0][nt][mt][i], acc[MATS - 1][nt][mt][i], limit, alpha));
+        } else {
+          const int token = pair / top, choice = pair - token * top;
+          out[((size_t)choice * tokens + token) * N + n] = with_extra(
+              acc[0][nt][mt][i] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
+        }
+      }
+  }
+}
+
 // Two groups of columns a wave from this many pairs on (the launch then still has blocks enough).
 #define WIDE_COLUMNS_MIN_PAIRS 1024
 
 // blocks of a launch: the items rounded up to a whole number a die
 static unsigned mfma_blocks(int slots, int column_tiles) { return (unsigned)(((long long)slots * column_tiles + 7) / 8 * 8); }
 
-// Which shape a launch takes: two column groups a wave from WIDE_COLUMNS_MIN_PAIRS pairs on, and blocks of 128
-// rows where an expert has at least two such tiles on average and K is 4,096 or more (measured, a prompt of
-// 2,048 tokens: at a width of 4,096 10.0 -> 9.7 ms, at 2,048 3.80 -> 3.89 ms).
+// Which shape a launch takes: from WIDE_COLUMNS_MIN_PAIRS pairs on the one whose weight tile goes through LDS
+// (a prompt of 2,048 tokens at a width of 2,048: 3.80 -> 3.67 ms against the direct shape with two column groups
+// a wave; at 4,096: 10.0 -> 9.6 ms, where the direct shape with blocks of 128 rows reached 9.9), below that the
+// direct shape with one column group a wave, which streams the weight at 3 to 4.7 TB/s in a decode step.
 #define MFMA_LAUNCH(MODE, COLUMNS, A, W, PW, ACT, OUT, N_, K_, LIMIT, ALPHA, EXTRA, EXTRA_PARTS)                          \
   do {                                                                                                                   \
-    const bool wide = pairs >= WIDE_COLUMNS_MIN_PAIRS, tall = wide && pairs / experts >= 256 && (K_) >= 4096;                             \
-    const int slots = (int)(pairs / (tall ? 128 : TM) + experts);                                                        \
+    const bool wide = pairs >= WIDE_COLUMNS_MIN_PAIRS;                                                                   \
+    const int slots = (int)(pairs / TM + experts);                                                                       \
     const int tiles = ((COLUMNS) + (wide ? 2 : 1) * TN - 1) / ((wide ? 2 : 1) * TN);                                      \
-    if (tall)                                                                                                            \
-      moe_grouped_mfma_kernel<MODE, 2, 8><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \
-          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
-    else if (wide)                                                                                                       \
-      moe_grouped_mfma_kernel<MODE, 2, 4><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \
+    if (wide)                                                                                                            \
+      moe_grouped_staged_kernel<MODE><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                    \
           A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
     else                                                                                                                 \
       moe_grouped_mfma_kernel<MODE, 1, 4><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \

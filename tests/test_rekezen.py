@@ -151,7 +151,7 @@ def test_rotary_tables():
     """Frequencies and magnitude against the plain table: a ramp inside the table, one that starts before
     it, one beyond it (every pair keeps its frequency), no scaling."""
     from forge_engine_amd.parts.rotary import RotaryPosition, YarnRotaryPosition
-    for dims, base, scaling in ((32, 50000.0, (4.0, 2048, 32.0, 1.0)), (8, 100.0, (8.0, 64, 16.0, 2.0)),
+    for dims, base, scaling in ((24, 20000.0, (6.0, 512, 24.0, 1.0)), (8, 100.0, (8.0, 64, 16.0, 2.0)),
                                 (16, 10000.0, (2.0, 1 << 20, 1.0, 0.5)), (12, 300.0, (3.0, 16, 64.0, 32.0))):
         rot = {"dims": dims, "base": base, "scaling": dict(zip(("factor", "original", "fast", "slow"), scaling))}
         part = YarnRotaryPosition(_ctx(), head_dim=dims + 4, theta=base, rotary_dim=dims, factor=scaling[0], original=scaling[1],

@@ -83,7 +83,7 @@ def test_token_pair_embedding_kernel(dtype):
     assert want_prev[:, 0].tolist() == [2, 7, 9, 69, 0]
 
 
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim,rot", [(4, 2, 16, 24, 8), (6, 3, 128, 128, 32), (2, 2, 12, 20, 12), (3, 1, 64, 8, 0)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,rot", [(4, 2, 16, 24, 8), (6, 2, 128, 128, 64), (2, 2, 12, 20, 12), (3, 1, 64, 8, 0)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_whole_norm_rope_write_kernel(heads, kv_heads, dim, vdim, rot, dtype):
     from forge_engine_amd.kernels import ops
@@ -114,7 +114,7 @@ def test_whole_norm_rope_write_kernel(heads, kv_heads, dim, vdim, rot, dtype):
         assert write_kv or not bool(got_k.any())
 
 
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 16, 24), (6, 3, 128, 128), (2, 2, 12, 20)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 16, 24), (8, 2, 128, 128), (2, 2, 12, 20)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_masked_attention_with_cap_and_head_gates(heads, kv_heads, dim, vdim, dtype):
     from forge_engine_amd.kernels import ops
@@ -143,7 +143,7 @@ def test_masked_attention_with_cap_and_head_gates(heads, kv_heads, dim, vdim, dt
     close(got, want, dtype)
 
 
-@pytest.mark.parametrize("tokens,hidden,experts,top,inner", [(1, 48, 5, 2, 20), (37, 64, 3, 1, 36), (150, 256, 8, 2, 64), (70, 40, 4, 4, 100)])
+@pytest.mark.parametrize("tokens,hidden,experts,top,inner", [(1, 48, 5, 2, 20), (37, 64, 3, 1, 36), (150, 256, 6, 2, 96), (70, 40, 4, 4, 100), (600, 128, 4, 2, 160)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mixture_of_experts_kernels(tokens, hidden, experts, top, inner, dtype):
     from forge_engine_amd.kernels import ops
