@@ -54,10 +54,11 @@ class DecoderModel:
 
     def ignorable_names(self) -> set[str]:
         """Tensors a checkpoint may hold that the model does not read: the head
-        matrix of a model whose head is tied to the embedding."""
+        matrix of a model whose head is tied to the embedding, and whatever the plan names."""
+        names = set(self.plan.ignorable_names) - set(self._specs)
         if getattr(self.head, "tied", False):
-            return {self.head.name(getattr(self.head, "leaf", "weight"))}
-        return set()
+            names.add(self.head.name(getattr(self.head, "leaf", "weight")))
+        return names
 
     def set_param(self, name: str, tensor: Tensor) -> None:
         self._owners[name].set_param(name, tensor)

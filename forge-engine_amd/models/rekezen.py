@@ -62,13 +62,15 @@ def rekezen_plan(config: RekezenConfig) -> ModelPlan:
     def norm(name: str) -> PartSpec:
         return PartSpec("layer_norm", {"size": width, "eps": eps, "leaf": "", "bias_leaf": "b"}, name)
 
-    layers, schedule = [], []
+    layers, schedule, unread = [], [], set()
     for index, layer in enumerate(config.layers):
         prefix = f"l{index}"
         feed_forward = _feed_forward(config, layer.get("mlp"), f"{prefix}.mlp")
         norms = {"input": norm(f"{prefix}.norm1")}
         if feed_forward is not None:
             norms["post_mixer"] = norm(f"{prefix}.norm2")
+        else:       # a checkpoint may still hold what a feed-forward's sublayer would have read
+            unread |= {f"{prefix}.norm2", f"{prefix}.norm2.b", f"{prefix}.hc2.in", f"{prefix}.hc2.out", f"{prefix}.hc2.mix"}
         if config.streams is None:
             arrangement, params = "pre_norm", {}
         else:
@@ -94,6 +96,7 @@ def rekezen_plan(config: RekezenConfig) -> ModelPlan:
         head=PartSpec("lm_head", dict(sizes, tied=True, scale=config.logit_scale), "embed"),
         eos_token_ids=frozenset() if config.eos_token_id is None else frozenset({config.eos_token_id}),
         max_positions=None,
+        ignorable_names=frozenset(unread),
     )
 
 

@@ -55,6 +55,7 @@ class ModelPlan:
     head: PartSpec
     eos_token_ids: frozenset = frozenset()
     max_positions: int | None = None
+    ignorable_names: frozenset = frozenset()   # tensors that a checkpoint may hold and the model does not read
 
     def resolved_schedule(self) -> tuple[LayerCall, ...]:
         """The run order with every cache slot made explicit and checked."""

@@ -267,3 +267,21 @@ def test_decoding_from_the_first_token(folders, tmp_path, monkeypatch):
     requests = requests_of("A", 8, (45,))
     got = ru.run_trace(folders["A"], "float32", ru.trace_tail(requests, 10 ** 6), tmp_path, block_size=4, device="cpu", on_cpu=True)
     ku.compare(got, ku.plain_logits(folders["A"], requests), "float32")
+
+
+def test_a_checkpoint_may_hold_the_norm_of_a_feed_forward_that_is_not_there(folders, tmp_path, monkeypatch):
+    """A layer without a feed-forward reads no second norm and no second set of stream weights; a
+    checkpoint that holds them all the same loads, and they change nothing."""
+    import json
+    import shutil
+    from safetensors.torch import load_file, save_file
+    kernel_refs.install(monkeypatch)
+    folder = shutil.copytree(folders["A"], tmp_path / "more")
+    weights = load_file(str(folder / "model.safetensors"))
+    assert "l1.norm2" not in weights
+    weights.update({"l1.norm2": torch.ones(48).bfloat16(), "l1.norm2.b": torch.ones(48).bfloat16(), "l1.hc2.in": torch.ones(3).bfloat16(),
+                    "l1.hc2.out": torch.ones(3).bfloat16(), "l1.hc2.mix": torch.ones(3, 3).bfloat16()})
+    save_file({n: t.contiguous() for n, t in weights.items()}, str(folder / "model.safetensors"))
+    requests = requests_of("A", 5, (9,))
+    got = ru.run_trace(folder, "float32", ru.trace_whole(requests), tmp_path / "out", block_size=4, device="cpu", on_cpu=True)
+    ku.compare(got, ku.plain_logits(folders["A"], requests), "float32")
