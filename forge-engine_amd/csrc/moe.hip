@@ -377,7 +377,9 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
 // the CU's L1 (measured: 80 million a launch, 312,000 a CU in 473,000 cycles, with the matrix cores busy 14 %);
 // here four neighbouring lanes bring 64 neighbouring bytes of one weight row, a quarter of the accesses, and every
 // wave reads its fragments out of LDS.  Block = 64 rows x 128 columns (MODE 0: and their 128 up columns), K in
-// steps of 32, two stages, operands requested DEPTH steps ahead, one LDS-only barrier a step.
+// steps of 32, two stages, operands requested DEPTH steps ahead, one LDS-only barrier a step.  (Rows of 64 bytes
+// with their 16-byte pieces exchanged by the row's number, instead of rows 80 bytes apart, took the bank conflicts
+// from 20 million cycles a launch to none and the launch from 179 to 181 us: they were not what it waits for.)
 template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_staged_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
@@ -461,9 +463,11 @@ __global__ __launch_bounds__(256) void moe_grouped_staged_kernel(
   for (; step + DEPTH <= steps; step += DEPTH) {
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u) {
+      // set u went into LDS during the step before: its registers are free, and what is asked for now has
+      // this step's products and the next step's to arrive in
+      fetch(step + u + DEPTH, u);
       multiply(u & 1);
       stash((u + 1) & 1, (u + 1) % DEPTH);
-      fetch(step + u + DEPTH, u);
       lds_barrier();
     }
   }
