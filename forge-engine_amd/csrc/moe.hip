@@ -10,10 +10,12 @@
 //                    also takes what every token gets beside its experts, a shared expert's output)
 //   fe_gated_act:    the same activation over a dense [T, 2F] product (a shared expert)
 //
-// The grouped products tile the sorted rows 32 at a time within an expert (a tile never spans two
-// experts) and 64 output columns a block, K through LDS in steps of 32, float32 FMA accumulation.
-// A launch has as many row-tile slots as the pairs could need at worst (pairs / 32 + experts);
-// a block whose slot lies beyond the tiles there are returns at once.
+// The grouped products tile the sorted rows within an expert (a tile never spans two experts).  float32, and
+// bfloat16 with K no multiple of 32: 32 rows x 64 columns a block, K through LDS in steps of 32, FMA.  bfloat16:
+// MFMA 16x16x32 over 64 rows x 64 columns with the weight straight into the operands (steps of few rows: a
+// decode step streams every expert's weight once), or 64 rows x 128 columns with the weight tile through LDS like
+// the rows (steps of many rows).  A launch has as many row-tile slots as the pairs could need at worst (pairs /
+// rows a tile + experts); a block whose slot lies beyond the tiles there are returns at once.
 #include "common.h"
 
 // One thread per token over its row of router logits z [T, E] (float32, the product comes from the
