@@ -381,7 +381,12 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
 // wave reads its fragments out of LDS.  Block = 64 rows x 128 columns (MODE 0: and their 128 up columns), K in
 // steps of 32, two stages, operands requested DEPTH steps ahead, one LDS-only barrier a step.  (Rows of 64 bytes
 // with their 16-byte pieces exchanged by the row's number, instead of rows 80 bytes apart, took the bank conflicts
-// from 20 million cycles a launch to none and the launch from 179 to 181 us: they were not what it waits for.)
+// from 20 million cycles a launch to none and the launch from 179 to 181 us: they were not what it waits for.
+// Rows and weight tile straight from global memory into LDS (`global_load_lds_dwordx4`, no staging registers,
+// three and four steps deep) gave 3.85 instead of 3.64 ms for a prompt of 2,048 tokens at a width of 2,048.  With
+// the products taken out of this kernel its loads, LDS stores and barriers alone take 124 of the 174 us, and with
+// every block reading the same hot tile 151: neither the depth of the prefetch nor where the bytes come from
+// is what bounds it.)
 template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_staged_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
